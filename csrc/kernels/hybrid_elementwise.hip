@@ -1,0 +1,279 @@
+// Row kernels of the hybrid (mixed attention / recurrent) model family, whose residual stream
+// and norms are fp32 while the GEMM operands keep the model's storage type.
+//
+// Every kernel is built for two storage types: bf16 (dt = 0, the serving format) and fp32
+// (dt = 1, the exact mode, where weights, GEMM operands and caches are all fp32). "S" below is
+// that storage type; residuals, projection outputs that feed a norm, a gate or a recurrence,
+// and all arithmetic are fp32 in both.
+//
+//  * embedding_f32      x[t] = table[ids[t]] as fp32 (two copies: the stream and the loop input)
+//  * resadd_groupnorm   x = keep * x + mult * y + bias; h = grouped RMS norm of x (S out)
+//  * concat_cast        [x ; x0] fp32 -> S rows of width 2D (the operand of the loop-entry GEMM)
+//  * gelu_mul           gelu_tanh(gate) * up over a [T, 2F] fp32 projection -> S [T, F]
+//  * attn_prepare       per-head RMS norm of q and k (shared weights), normed k -> key cache,
+//                       raw k -> value cache ("values are the keys"), normed q -> S
+//  * mla_prepare        latent attention: RMS norm of the compressed kv -> cache, interleaved
+//                       rotary on the shared rotated key -> cache, rotary on each head's rotated
+//                       query part; the unrotated query parts go to a GEMM operand
+#include "common.h"
+
+namespace {
+
+template <typename S> __device__ __forceinline__ float ldf(const S* p);
+template <> __device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename S> __device__ __forceinline__ void stf(S* p, float v);
+template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+template <typename S>
+__global__ void __launch_bounds__(256) embedding_f32_kernel(
+    float* __restrict__ x, float* __restrict__ x0, const int* __restrict__ ids,
+    const S* __restrict__ table, int T, int dim, int vocab) {
+  const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (long)T * dim) return;
+  const int t = (int)(gid / dim), c = (int)(gid % dim);
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const float v = ldf(table + (long)id * dim + c);
+  x[gid] = v;
+  if (x0 != nullptr) x0[gid] = v;
+}
+
+// One workgroup per row. x (fp32, in place): x = keep * x + mult * y + bias, y and bias may be
+// null. The row is cut into `groups` equal parts, each scaled by its own rsqrt(mean(sq) + eps);
+// h = that * w. h may be null (the last layer's add). rows_idx (nullable) selects source rows
+// (the final norm of the rows whose logits are wanted); it excludes y / bias / the write-back.
+template <typename S>
+__global__ void __launch_bounds__(256) resadd_groupnorm_kernel(
+    float* __restrict__ x, const float* __restrict__ y, int ldy, const S* __restrict__ bias,
+    float keep, float mult, const S* __restrict__ w, S* __restrict__ h, int ldh, int dim,
+    int groups, float eps, const long* __restrict__ rows_idx) {
+  extern __shared__ float row[];            // dim floats + groups partial sums
+  float* gsum = row + dim;
+  const int r = blockIdx.x;
+  const long src = rows_idx ? rows_idx[r] : r;
+  float* xr = x + src * dim;
+  for (int g = threadIdx.x; g < groups; g += blockDim.x) gsum[g] = 0.f;
+  for (int c = threadIdx.x; c < dim; c += blockDim.x) {
+    float v = xr[c];
+    if (rows_idx == nullptr) {
+      v = keep != 0.f ? v * keep : 0.f;
+      if (y != nullptr) v += mult * y[(long)r * ldy + c];
+      if (bias != nullptr) v += ldf(bias + c);
+      if (y != nullptr || bias != nullptr || keep != 1.f) xr[c] = v;
+    }
+    row[c] = v;
+  }
+  __syncthreads();
+  if (h == nullptr) return;
+  const int gl = dim / groups;
+  // one wave per group, in turn: a wave sums its group's squares in a fixed order
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int g = wid; g < groups; g += nw) {
+    float s = 0.f;
+    for (int c = lane; c < gl; c += 64) { const float v = row[g * gl + c]; s += v * v; }
+    s = wave_sum(s);
+    if (lane == 0) gsum[g] = 1.f / sqrtf(s / (float)gl + eps);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < dim; c += blockDim.x)
+    stf(h + (long)r * ldh + c, row[c] * gsum[c / gl] * ldf(w + c));
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) concat_cast_kernel(
+    S* __restrict__ out, const float* __restrict__ a, const float* __restrict__ b, int T,
+    int dim) {
+  const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (long)T * 2 * dim) return;
+  const int t = (int)(gid / (2 * dim)), c = (int)(gid % (2 * dim));
+  stf(out + gid, c < dim ? a[(long)t * dim + c] : b[(long)t * dim + c - dim]);
+}
+
+__device__ __forceinline__ float gelu_tanh32(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) gelu_mul_kernel(
+    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F) {
+  const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (long)T * F) return;
+  const int t = (int)(gid / F), c = (int)(gid % F);
+  const float* r = gu + (long)t * ldg;
+  stf(out + (long)t * ldo + c, gelu_tanh32(r[c]) * r[F + c]);
+}
+
+// proj row: [H*d q | G*d k | ...]; one wave per (token, head) unit, H + G units per token.
+template <typename S>
+__global__ void __launch_bounds__(256) attn_prepare_kernel(
+    const float* __restrict__ proj, int ldp, const S* __restrict__ qw, const S* __restrict__ kw,
+    float eps, int T, int H, int G, int d, S* __restrict__ q_out, S* __restrict__ kcache,
+    S* __restrict__ vcache, const int* __restrict__ slots) {
+  const int lane = threadIdx.x & 63;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= (long)T * (H + G)) return;
+  const int t = (int)(unit / (H + G)), u = (int)(unit % (H + G));
+  const bool is_q = u < H;
+  const float* src = proj + (long)t * ldp + (is_q ? u * d : H * d + (u - H) * d);
+  float s = 0.f;
+  for (int c = lane; c < d; c += 64) { const float v = src[c]; s += v * v; }
+  s = wave_sum(s);
+  const float rs = 1.f / sqrtf(s / (float)d + eps);
+  if (is_q) {
+    S* dst = q_out + ((long)t * H + u) * d;
+    for (int c = lane; c < d; c += 64) stf(dst + c, src[c] * rs * ldf(qw + c));
+  } else {
+    const int slot = slots[t];
+    if (slot < 0) return;
+    const int g = u - H;
+    S* kd = kcache + ((long)slot * G + g) * d;
+    S* vd = vcache + ((long)slot * G + g) * d;
+    for (int c = lane; c < d; c += 64) {
+      const float v = src[c];
+      stf(kd + c, v * rs * ldf(kw + c));
+      stf(vd + c, v);
+    }
+  }
+}
+
+// proj row: [H*(d+dr) q | r compressed kv | dr shared rotated key]. One workgroup per token.
+//  cache row (width r + dr): [normed latent | rotated key]
+//  q_nope [T, H, d] (S): operand of the per-head absorb GEMM
+//  q_full [T, H, r + dr] (S): this kernel writes the rotated tail [r, r+dr) of every head
+// inv_freq [rot_dims / 2] fp32; pairs (2i, 2i+1) of the first rot_dims of the dr part rotate.
+template <typename S>
+__global__ void __launch_bounds__(256) mla_prepare_kernel(
+    const float* __restrict__ proj, int ldp, const S* __restrict__ cw, float eps, int T, int H,
+    int d, int dr, int r, int rot_dims, const float* __restrict__ inv_freq,
+    const int* __restrict__ positions, const int* __restrict__ slots, S* __restrict__ q_nope,
+    S* __restrict__ q_full, S* __restrict__ cache) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  const float* row = proj + (long)t * ldp;
+  const float* dkv = row + (long)H * (d + dr);
+  const float pos = (float)positions[t];
+  const int slot = slots[t];
+  float s = 0.f;
+  for (int c = threadIdx.x; c < r; c += blockDim.x) { const float v = dkv[c]; s += v * v; }
+  s = block_sum(s, red);
+  const float rs = 1.f / sqrtf(s / (float)r + eps);
+  if (slot >= 0) {
+    S* cr = cache + (long)slot * (r + dr);
+    for (int c = threadIdx.x; c < r; c += blockDim.x) stf(cr + c, dkv[c] * rs * ldf(cw + c));
+    for (int c = threadIdx.x; c < dr; c += blockDim.x) {
+      float v = dkv[r + c];
+      if (c < rot_dims) {
+        const float a = pos * inv_freq[c >> 1];
+        const float cs = cosf(a), sn = sinf(a);
+        const float o = dkv[r + (c ^ 1)];
+        v = (c & 1) ? v * cs + o * sn : v * cs - o * sn;
+      }
+      stf(cr + r + c, v);
+    }
+  }
+  for (int i = threadIdx.x; i < H * (d + dr); i += blockDim.x) {
+    const int h = i / (d + dr), c = i % (d + dr);
+    float v = row[i];
+    if (c < d) {
+      stf(q_nope + ((long)t * H + h) * d + c, v);
+    } else {
+      const int cc = c - d;
+      if (cc < rot_dims) {
+        const float a = pos * inv_freq[cc >> 1];
+        const float cs = cosf(a), sn = sinf(a);
+        const float o = row[h * (d + dr) + d + (cc ^ 1)];
+        v = (cc & 1) ? v * cs + o * sn : v * cs - o * sn;
+      }
+      stf(q_full + ((long)t * H + h) * (r + dr) + r + cc, v);
+    }
+  }
+}
+
+}  // namespace
+
+#define DT_SWITCH(dt, CALL_BF16, CALL_F32) \
+  do {                                     \
+    if ((dt) == 0) { CALL_BF16; }          \
+    else if ((dt) == 1) { CALL_F32; }      \
+    else return (int)hipErrorInvalidValue; \
+  } while (0)
+
+extern "C" int dli_embedding_f32(float* x, float* x0, const int* ids, const void* table, int T,
+                                 int dim, int vocab, int dt, hipStream_t st) {
+  if (T <= 0) return 0;
+  const int nb = (int)(((long)T * dim + 255) / 256);
+  DT_SWITCH(dt,
+            (embedding_f32_kernel<u16><<<nb, 256, 0, st>>>(x, x0, ids, (const u16*)table, T, dim, vocab)),
+            (embedding_f32_kernel<float><<<nb, 256, 0, st>>>(x, x0, ids, (const float*)table, T, dim, vocab)));
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_resadd_groupnorm(float* x, const float* y, int ldy, const void* bias,
+                                    float keep, float mult, const void* w, void* h, int ldh,
+                                    int rows, int dim, int groups, float eps,
+                                    const long* rows_idx, int dt, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (groups < 1 || dim % groups || (size_t)(dim + groups) * 4 > 60000)
+    return (int)hipErrorInvalidValue;
+  const size_t sh = (size_t)(dim + groups) * 4;
+  DT_SWITCH(dt,
+            (resadd_groupnorm_kernel<u16><<<rows, 256, sh, st>>>(
+                x, y, ldy, (const u16*)bias, keep, mult, (const u16*)w, (u16*)h, ldh, dim, groups,
+                eps, rows_idx)),
+            (resadd_groupnorm_kernel<float><<<rows, 256, sh, st>>>(
+                x, y, ldy, (const float*)bias, keep, mult, (const float*)w, (float*)h, ldh, dim,
+                groups, eps, rows_idx)));
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_concat_cast(void* out, const float* a, const float* b, int T, int dim, int dt,
+                               hipStream_t st) {
+  if (T <= 0) return 0;
+  const int nb = (int)(((long)T * 2 * dim + 255) / 256);
+  DT_SWITCH(dt, (concat_cast_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, a, b, T, dim)),
+            (concat_cast_kernel<float><<<nb, 256, 0, st>>>((float*)out, a, b, T, dim)));
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_gelu_mul(void* out, int ldo, const float* gu, int ldg, int T, int F, int dt,
+                            hipStream_t st) {
+  if (T <= 0) return 0;
+  const int nb = (int)(((long)T * F + 255) / 256);
+  DT_SWITCH(dt, (gelu_mul_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F)),
+            (gelu_mul_kernel<float><<<nb, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F)));
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_attn_prepare(const float* proj, int ldp, const void* qw, const void* kw,
+                                float eps, int T, int H, int G, int d, void* q_out, void* kcache,
+                                void* vcache, const int* slots, int dt, hipStream_t st) {
+  if (T <= 0) return 0;
+  const long units = (long)T * (H + G);
+  const int nb = (int)((units + 3) / 4);
+  DT_SWITCH(dt,
+            (attn_prepare_kernel<u16><<<nb, 256, 0, st>>>(
+                proj, ldp, (const u16*)qw, (const u16*)kw, eps, T, H, G, d, (u16*)q_out,
+                (u16*)kcache, (u16*)vcache, slots)),
+            (attn_prepare_kernel<float><<<nb, 256, 0, st>>>(
+                proj, ldp, (const float*)qw, (const float*)kw, eps, T, H, G, d, (float*)q_out,
+                (float*)kcache, (float*)vcache, slots)));
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_mla_prepare(const float* proj, int ldp, const void* cw, float eps, int T,
+                               int H, int d, int dr, int r, int rot_dims, const float* inv_freq,
+                               const int* positions, const int* slots, void* q_nope,
+                               void* q_full, void* cache, int dt, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot_dims > dr || (rot_dims & 1)) return (int)hipErrorInvalidValue;
+  DT_SWITCH(dt,
+            (mla_prepare_kernel<u16><<<T, 256, 0, st>>>(
+                proj, ldp, (const u16*)cw, eps, T, H, d, dr, r, rot_dims, inv_freq, positions,
+                slots, (u16*)q_nope, (u16*)q_full, (u16*)cache)),
+            (mla_prepare_kernel<float><<<T, 256, 0, st>>>(
+                proj, ldp, (const float*)cw, eps, T, H, d, dr, r, rot_dims, inv_freq, positions,
+                slots, (float*)q_nope, (float*)q_full, (float*)cache)));
+  DLI_RETURN_LAUNCH();
+}

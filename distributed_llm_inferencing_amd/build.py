@@ -49,8 +49,11 @@ def _hipcc() -> str:
 
 # NOTE: no -ffast-math: it implies no-infs, and the attention/sampling kernels rely on
 # -inf as the masked-score / running-max sentinel (poison under ninf -> NaNs).
+# packed-fp32-ops off: hipcc -O3 pairs ordinary float code into v_pk_*_f32 by itself, and
+# some forms of those have returned wrong values on this hardware without any error
 KERNEL_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc",
-                "-munsafe-fp-atomics", "-Wno-unused-result"]
+                "-munsafe-fp-atomics", "-Wno-unused-result",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 RUNTIME_FLAGS = ["-O2", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wall",
                  "-Wno-unused-result"]
 

@@ -54,6 +54,11 @@ class StepMeta:
     packed_payload: Optional[np.ndarray] = None
     table_width_full: int = 0
     core: Optional[tuple] = None
+    # recurrent-state slot of each sequence (models with per-sequence state; not on the wire)
+    state_slots: Optional[np.ndarray] = None
+    # rows (token indices of this step) whose logits are wanted instead of sampled tokens
+    # (trace replay / scoring; not on the wire)
+    logit_rows: Optional[np.ndarray] = None
 
     @property
     def num_seqs(self) -> int:
@@ -195,6 +200,8 @@ class DeviceBatch:
     max_context_decode: int = 0
     cu_seqlens_prefill: Optional[torch.Tensor] = None
     max_seqlen_prefill: int = 0
+    state_slots: Optional[torch.Tensor] = None
+    logit_rows: Optional[torch.Tensor] = None
 
     @property
     def is_prefill(self) -> bool:
@@ -231,6 +238,8 @@ def to_device(meta: StepMeta, device, pin: bool = True) -> DeviceBatch:
     add("top_k", meta.top_k, torch.int32)
     add("top_p", meta.top_p, torch.float32)
     add("seeds", meta.seeds, torch.int64)
+    add("state_slots", meta.state_slots, torch.int32)
+    add("logit_rows", meta.logit_rows, torch.int64)
     nd = int(meta.num_decode) if meta.kind == PREFILL else 0
     paged = False
     if meta.kind == PREFILL:
@@ -266,7 +275,8 @@ def to_device(meta: StepMeta, device, pin: bool = True) -> DeviceBatch:
     db = DeviceBatch(kind=meta.kind, num_seqs=S, num_tokens=T,
                      input_ids=v.get("input_ids"), positions=v.get("positions"),
                      slot_mapping=v.get("slot_mapping"), temperature=v.get("temperature"),
-                     top_k=v.get("top_k"), top_p=v.get("top_p"), seeds=v.get("seeds"))
+                     top_k=v.get("top_k"), top_p=v.get("top_p"), seeds=v.get("seeds"),
+                     state_slots=v.get("state_slots"), logit_rows=v.get("logit_rows"))
     if meta.kind == PREFILL:
         db.cu_seqlens = v["cu_seqlens"]
         db.max_seqlen = int(lens.max()) if S else 0

@@ -17,6 +17,8 @@ from ..models.configs import ModelConfig
 
 
 def bytes_per_block(cfg: ModelConfig, num_layers: int, block_size: int, dtype_bytes: int = 2):
+    if cfg.is_hybrid:
+        return max(1, cfg.kv_bytes_per_token(dtype_bytes)) * block_size
     return 2 * num_layers * cfg.num_kv_heads * cfg.head_dim * block_size * dtype_bytes
 
 
@@ -81,3 +83,80 @@ class KVCache:
     @property
     def capacity_tokens(self) -> int:
         return self.num_blocks * self.block_size
+
+
+class HybridCache:
+    """Caches and recurrent states of a hybrid design, one entry per layer run (a looped layer
+    has one per pass), all addressed by the engine's one block manager / state-slot manager:
+
+    * ``attention``:        (k [slots, G*d], v [slots, G*d])   token-major rows, slot =
+                            block * block_size + offset; k holds the normed keys, v the raw ones
+    * ``latent_attention``: (c [slots, kv_rank + rot_dim],)     normed latent | rotated key
+    * ``hgrn2``:            (state [state_slots, H, d, dv] fp32,)  one slot per live sequence
+
+    Rows are zero-initialised once (padding rows of captured decode steps read row 0). A state
+    slot is not cleared on reuse: a sequence's first portion starts from zero by position."""
+
+    def __init__(self, cfg: ModelConfig, num_blocks: int, block_size: int, state_slots: int,
+                 device, dtype=torch.bfloat16):
+        self.cfg = cfg
+        self.num_blocks = num_blocks
+        self.block_size = block_size
+        self.state_slots = state_slots
+        self.num_layers = len(cfg.layer_runs())
+        rows = num_blocks * block_size
+        self.entries = []
+        for li, _, _ in cfg.layer_runs():
+            s = cfg.layer_specs[li]
+            if s.kind == "attention":
+                e = (torch.zeros(rows, s.kv_heads * s.dim, dtype=dtype, device=device),
+                     torch.zeros(rows, s.kv_heads * s.dim, dtype=dtype, device=device))
+            elif s.kind == "latent_attention":
+                e = (torch.zeros(rows, s.kv_rank + s.rot_dim, dtype=dtype, device=device),)
+            else:
+                e = (torch.zeros(state_slots, s.heads, s.dim, s.vdim, dtype=torch.float32,
+                                 device=device),)
+            self.entries.append(e)
+
+    def layers(self) -> "HybridCache":
+        """What the runner hands to the model: the cache itself (entries + block size)."""
+        return self
+
+    @property
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for e in self.entries for t in e)
+
+    @property
+    def capacity_tokens(self) -> int:
+        return self.num_blocks * self.block_size
+
+
+class StateSlots:
+    """Recurrent-state slots of the live sequences: a free list over ``num_slots`` rows of the
+    state tensors (``HybridCache``). A sequence takes a slot when it is admitted and gives it
+    back when it finishes or is preempted; slots are reused without clearing."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = int(num_slots)
+        self._free = list(range(self.num_slots - 1, -1, -1))
+        self._of: dict = {}
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def get(self, seq_id: int) -> int:
+        return self._of.get(seq_id, -1)
+
+    def acquire(self, seq_id: int) -> int:
+        s = self._of.get(seq_id)
+        if s is None:
+            if not self._free:
+                return -1
+            s = self._of[seq_id] = self._free.pop()
+        return s
+
+    def release(self, seq_id: int) -> None:
+        s = self._of.pop(seq_id, None)
+        if s is not None:
+            self._free.append(s)

@@ -17,10 +17,11 @@ import numpy as np
 import torch
 
 from ..models.configs import ModelConfig, get_config
+from ..models import model_class
 from ..models.model import TransformerLM
 from ..runtime import BlockManager
 from ..tokenizer import load_tokenizer
-from .kv_cache import KVCache, auto_num_blocks
+from .kv_cache import HybridCache, KVCache, StateSlots, auto_num_blocks
 from .runner import StageRunner
 from .scheduler import Scheduler
 from .sequence import RequestOutput, SamplingParams, Sequence
@@ -111,16 +112,24 @@ class LLMEngine:
         if lm is not None:
             self.model = lm
         elif params is None:
-            self.model = TransformerLM.random(cfg, device=self.device, dtype=dtype, seed=seed)
+            self.model = model_class(cfg).random(cfg, device=self.device, dtype=dtype, seed=seed)
         else:
-            self.model = TransformerLM(cfg, {k: v.to(self.device) for k, v in params.items()},
-                                       device=self.device)
+            self.model = model_class(cfg)(cfg, {k: v.to(self.device) for k, v in params.items()},
+                                          device=self.device)
         max_model_len = min(max_model_len, cfg.max_position)
         if num_blocks is None:
             # KV pool sized from free HBM, optionally capped
             num_blocks = auto_num_blocks(cfg, cfg.num_layers, block_size, self.device,
                                          kv_fraction, cap_tokens=max_kv_tokens or 0)
-        self.kv = KVCache(cfg, cfg.num_layers, num_blocks, block_size, self.device, dtype)
+        self.state_slots = None
+        if cfg.is_hybrid:
+            # one cache / state entry per layer run; a recurrent-state slot per live sequence
+            dtype = getattr(self.model, "dtype", dtype)
+            self.kv = HybridCache(cfg, num_blocks, block_size, max_batch, self.device, dtype)
+            if cfg.has_state:
+                self.state_slots = StateSlots(max_batch)
+        else:
+            self.kv = KVCache(cfg, cfg.num_layers, num_blocks, block_size, self.device, dtype)
         self.bm = BlockManager(num_blocks, block_size)
         # mixed prefill+decode steps (DLI_MIXED_STEPS=0 = off); engines in lockstep with peer
         # ranks (EP / TP) pass False so every rank's step kinds stay aligned
@@ -129,7 +138,10 @@ class LLMEngine:
         self.scheduler = Scheduler(self.bm, max_seqs_per_mb=max_batch,
                                    max_prefill_tokens=max_prefill_tokens,
                                    eos_token_id=cfg.eos_token_id, max_model_len=max_model_len,
-                                   mixed_steps=self.mixed_steps)
+                                   mixed_steps=self.mixed_steps, state_slots=self.state_slots,
+                                   always_paged=getattr(self.model, "needs_block_tables", False),
+                                   # cached KV blocks do not hold a recurrent state
+                                   prefix_caching=False if cfg.has_state else None)
         self.runner = StageRunner(self.model, self.kv, max_batch, self.scheduler.table_width,
                                   use_graphs=use_graphs)
         self.tokenizer = load_tokenizer(cfg, tokenizer_path)
@@ -237,6 +249,26 @@ class LLMEngine:
             self.spans.record(o)
             outs.append(o)
         return outs
+
+    def replay_step(self, entries, want=None, end=()) -> torch.Tensor:
+        """Run one step dictated from outside (``Scheduler.replay_step``): ``entries`` =
+        [(request id, next token ids)], ``want`` = per entry the indices among those tokens
+        whose logits are returned ([n_wanted, vocab] fp32, in entry order); ``end`` = requests
+        whose blocks and state slot are given back after the step. Nothing is sampled."""
+        if self._inflight is not None or self.scheduler.has_work():
+            raise RuntimeError("replay_step on an engine with generation requests in flight")
+        n_want = sum(len(w) for w in (want or []))
+        meta = self.scheduler.replay_step(entries, want)
+        if n_want == 0:
+            meta.logit_rows = np.zeros(1, np.int64)      # the step still runs; row discarded
+        with trace_range(f"engine.replay[{meta.num_seqs}]"), self.timer.phase("run_prefill"):
+            logits = self.runner.run(meta)
+        self.stats.steps += 1
+        self.stats.prefill_steps += 1
+        self.stats.prompt_tokens += meta.num_tokens
+        for rid in end:
+            self.scheduler.end_replay(rid)
+        return logits[:n_want]
 
     def generate(self, prompts: Iterable[Union[str, List[int]]],
                  params: Optional[SamplingParams] = None) -> List[RequestOutput]:

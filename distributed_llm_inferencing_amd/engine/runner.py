@@ -64,7 +64,7 @@ class StageRunner:
         self._off = {}
         o = 0
         for name, n in (("seeds", 2 * B), ("ids", B), ("pos", B), ("slots", B), ("ctx", B),
-                        ("temp", B), ("topk", B), ("topp", B), ("src", B),
+                        ("temp", B), ("topk", B), ("topp", B), ("src", B), ("sslot", B),
                         ("tables", B * W)):
             self._off[name] = (o, n)
             o += n
@@ -107,7 +107,8 @@ class StageRunner:
                            max_context=self.W * self.kv.block_size,
                            temperature=self._view("temp", b, torch.float32),
                            top_k=self._view("topk", b), top_p=self._view("topp", b, torch.float32),
-                           seeds=self._view("seeds", b, torch.int64))
+                           seeds=self._view("seeds", b, torch.int64),
+                           state_slots=self._view("sslot", b))
 
     def _fill_host(self, meta: StepMeta, b: int):
         j = self._slot = (self._slot + 1) % HOST_RING
@@ -138,6 +139,8 @@ class StageRunner:
         put("topp", meta.top_p.astype(np.float32), np.float32(1.0).view(np.int32))
         put("seeds", meta.seeds.astype(np.int64), 0)
         put("src", meta.feed_src if meta.feed_src is not None else np.full(S, -1, np.int32), -1)
+        put("sslot", meta.state_slots if meta.state_slots is not None
+            else np.full(S, -1, np.int32), -1)
         o, _ = self._off["tables"]
         tb = np.asarray(meta.block_tables, dtype=np.int32)
         if tb.shape[1] != self.W:
@@ -180,6 +183,8 @@ class StageRunner:
         """(shapes, weights) of every projection GEMM a decode step of M rows runs here."""
         from ..ops import gemm as G
         m = self.model
+        if m.cfg.is_hybrid:
+            return m.gemm_shapes(M)
         shapes, weights = [], {}
         lp = m.layers[0] if m.layers else {}
 
@@ -247,9 +252,9 @@ class StageRunner:
         for b in (buckets or self.buckets):
             shapes, weights = self.gemm_shapes(b)
             c = m.cfg
-            qkv = ((c.num_heads, c.num_kv_heads, c.head_dim) if c.arch != "gpt2" else None)
+            qkv = ((c.num_heads, c.num_kv_heads, c.head_dim) if c.arch == "llama" else None)
             normed = ()
-            if (b <= G.GEMV_MAX_M and G.DEFER_NORM and not c.is_moe and c.arch != "gpt2"
+            if (b <= G.GEMV_MAX_M and G.DEFER_NORM and not c.is_moe and c.arch == "llama"
                     and m.tp_reduce is None and m.layers):
                 lp = m.layers[0]           # batch-1 QKV and gate/up read a deferred norm
                 normed = {(lp["wqkv"].shape[0], lp["wqkv"].shape[1], "splitk"),
@@ -276,7 +281,7 @@ class StageRunner:
             log = lambda m: print(m, file=sys.stderr, flush=True)  # noqa: E731
         top = G._bucket(max(max_tokens, 2048))
         c = self.model.cfg
-        qkv = (c.num_heads, c.num_kv_heads, c.head_dim) if c.arch != "gpt2" else None
+        qkv = (c.num_heads, c.num_kv_heads, c.head_dim) if c.arch == "llama" else None
         b = 2048
         with self.tune_lock():
             while b <= top:
@@ -314,7 +319,7 @@ class StageRunner:
             torch.cuda.synchronize(self.device)      # no staged upload still reads the buffer
             h = self._host_np
             h[:] = 0
-            for name, pad in (("slots", -1), ("topk", 1)):
+            for name, pad in (("slots", -1), ("topk", 1), ("sslot", -1)):
                 o, n = self._off[name]
                 h[o:o + n] = pad
             self.meta_dev.copy_(self.meta_host)

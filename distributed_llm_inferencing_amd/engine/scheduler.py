@@ -158,8 +158,16 @@ class Scheduler:
                  table_width: Optional[int] = None, native_decode: bool = False,
                  admit_window_s: Optional[float] = None, admit_min_frac: float = 0.125,
                  refill_interval_s: Optional[float] = None,
-                 prefix_caching: Optional[bool] = None, mixed_steps: bool = False):
+                 prefix_caching: Optional[bool] = None, mixed_steps: bool = False,
+                 state_slots=None, always_paged: bool = False):
         self.bm = block_manager
+        # models with a recurrent state per sequence: a slot per admitted sequence
+        # (engine.kv_cache.StateSlots), released with the sequence's blocks
+        self.state_slots = state_slots
+        # models that attend through the paged cache in every step kind get block tables
+        # (and context lengths) on whole-prompt prefill steps too
+        self.always_paged = bool(always_paged)
+        self._replay: Dict[str, Sequence] = {}
         self.bs = block_manager.block_size
         self.max_seqs = max_seqs_per_mb
         self.max_prefill_tokens = max_prefill_tokens
@@ -290,6 +298,8 @@ class Scheduler:
         seq.finish_time = time.perf_counter()
         if free:
             self.bm.free(seq.seq_id)
+        if self.state_slots is not None:
+            self.state_slots.release(seq.seq_id)
         if seq.params.timeout_s is not None:
             self._deadlines -= 1
         self.finished.append(seq)
@@ -312,6 +322,8 @@ class Scheduler:
         victim = max(r, key=lambda s: s.arrival)
         r.remove(victim)
         self.bm.free(victim.seq_id)
+        if self.state_slots is not None:
+            self.state_slots.release(victim.seq_id)
         victim.state = SeqState.WAITING
         victim.num_prefilled = 0
         victim.num_preemptions += 1
@@ -319,6 +331,16 @@ class Scheduler:
         self.num_preempted += 1
         self.waiting.appendleft(victim)
         return True
+
+    def _slots_of(self, seqs) -> Optional[np.ndarray]:
+        """State slot of each sequence (acquired at its first step), None without slots."""
+        if self.state_slots is None:
+            return None
+        out = np.fromiter((self.state_slots.acquire(s.seq_id) for s in seqs), np.int32,
+                          len(seqs))
+        if (out < 0).any():
+            raise RuntimeError("no free recurrent-state slot (more live sequences than slots)")
+        return out
 
     def _sampling_arrays(self, seqs: List[Sequence]):
         n = len(seqs)
@@ -387,6 +409,8 @@ class Scheduler:
                         seeds=cat([dec.seeds, pre.seeds]), microbatch=mb, step_id=pre.step_id,
                         seq_ids_arr=sid)
         meta.num_decode = nd
+        if dec.state_slots is not None:
+            meta.state_slots = cat([dec.state_slots, pre.state_slots])
         if dec.feed_src is not None:
             meta.feed_src = cat([dec.feed_src, np.full(int(pre.num_tokens), -1, np.int32)])
         if pre.sample_mask is not None:
@@ -539,7 +563,7 @@ class Scheduler:
         pos = (np.arange(T, dtype=np.int32) - np.repeat(cu - starts, lens)).astype(np.int32)
         slots = self.bm.slot_mapping(sid, starts, lens)
         ctx = starts + lens
-        if chunked or mixed:
+        if chunked or mixed or self.always_paged:
             width = -(-max(s.total_len for s in picked) // self.bs)   # blocks held per seq
             tables = self.bm.fill_tables(sid.tolist(), width)
         else:
@@ -551,6 +575,7 @@ class Scheduler:
                         seeds=seeds, microbatch=mb, step_id=self._step, seq_ids_arr=sid)
         if not final.all():
             meta.sample_mask = final
+        meta.state_slots = self._slots_of(picked)
         return meta
 
     def _mb_state(self, mb: int, native: bool = False):
@@ -658,7 +683,76 @@ class Scheduler:
         meta.seq_ids_arr = sid
         if (feed >= 0).any():
             meta.feed_src = feed
+        if self.state_slots is not None:
+            meta.state_slots = self._slots_of([st.seqs[i] for i in idx.tolist()])
         return meta
+
+    # ------------------------------------------------------------------ replay
+    def replay_step(self, entries, want=None) -> StepMeta:
+        """A step dictated from outside (trace replay, scoring): ``entries`` = [(request id,
+        its next token ids)], all run as one batch — prompt portions of any length beside
+        single tokens. A request is admitted at its first entry (blocks and, for stateful
+        models, a state slot), may skip steps, and keeps what it holds until ``end_replay``.
+        ``want`` = per entry, the indices among its new tokens whose logits are wanted; nothing
+        is sampled. Same block manager, slot mapping, block tables and StepMeta as every
+        other step."""
+        self._step += 1
+        picked, starts_l, lens_l = [], [], []
+        for rid, toks in entries:
+            toks = [int(t) for t in toks]
+            if not toks:
+                raise ValueError(f"replay entry '{rid}' brings no tokens")
+            seq = self._replay.get(rid)
+            if seq is None:
+                seq = Sequence(seq_id=self._next_id, request_id=rid, prompt_ids=[],
+                               params=SamplingParams(max_new_tokens=0, ignore_eos=True))
+                self._next_id += 1
+                seq.state = SeqState.PREFILLING
+                self._replay[rid] = self.seqs[seq.seq_id] = seq
+            if seq in picked:
+                raise ValueError(f"replay request '{rid}' appears twice in one step")
+            seq.prompt_ids.extend(toks)
+            if not self.bm.ensure(seq.seq_id, seq.total_len):
+                raise RuntimeError(f"cache pool exhausted at request '{rid}' "
+                                   f"({seq.total_len} tokens, {self.bm.num_free} blocks free)")
+            picked.append(seq)
+            starts_l.append(seq.num_prefilled)
+            lens_l.append(len(toks))
+            seq.num_prefilled = seq.total_len
+        S = len(picked)
+        sid = np.fromiter((s.seq_id for s in picked), np.int64, S)
+        starts = np.asarray(starts_l, np.int32)
+        lens = np.asarray(lens_l, np.int32)
+        T = int(lens.sum())
+        ids = np.fromiter(itertools.chain.from_iterable(
+            s.prompt_ids[st:st + n] for s, st, n in zip(picked, starts_l, lens_l)), np.int32, T)
+        cu = np.zeros(S, np.int32)
+        cu[1:] = np.cumsum(lens)[:-1]
+        pos = (np.arange(T, dtype=np.int32) - np.repeat(cu - starts, lens)).astype(np.int32)
+        width = -(-max(s.total_len for s in picked) // self.bs)
+        temp, topk, topp, seeds = self._sampling_arrays(picked)
+        meta = StepMeta(kind=PREFILL, seq_ids=sid.tolist(), input_ids=ids, positions=pos,
+                        slot_mapping=self.bm.slot_mapping(sid, starts, lens), seq_lens=lens,
+                        context_lens=starts + lens,
+                        block_tables=self.bm.fill_tables(sid.tolist(), width), temperature=temp,
+                        top_k=topk, top_p=topp, seeds=seeds, step_id=self._step,
+                        seq_ids_arr=sid)
+        meta.sample_mask = np.zeros(S, np.bool_)
+        meta.state_slots = self._slots_of(picked)
+        rows = [int(cu[i]) + int(k) for i, w in enumerate(want or []) for k in w]
+        if any(not 0 <= k < lens_l[i] for i, w in enumerate(want or []) for k in w):
+            raise ValueError("wanted index outside its entry's tokens")
+        meta.logit_rows = np.asarray(rows, np.int64)
+        return meta
+
+    def end_replay(self, request_id: str) -> None:
+        """Give back the blocks and the state slot of a replayed request."""
+        seq = self._replay.pop(request_id, None)
+        if seq is not None:
+            self._finish(seq, "replay")
+            self.seqs.pop(seq.seq_id, None)
+            if seq in self.finished:
+                self.finished.remove(seq)
 
     # ------------------------------------------------------------------ results
     def update(self, meta: StepMeta, tokens) -> List[Sequence]:

@@ -14,9 +14,36 @@ from typing import Optional
 
 
 @dataclass(frozen=True)
+class LayerSpec:
+    """One layer of a hybrid (layer-list) design: which sequence mixer it has, the mixer's
+    sizes and constants, and its feed-forward width (0 = none).
+
+    kinds: ``attention`` (windowed softmax attention, values = the un-normed keys, linear
+    distance bias, head mixing, output gate), ``hgrn2`` (gated linear recurrence with a
+    [dim, vdim] state per head) and ``latent_attention`` (keys / values expanded from a cached
+    low-rank latent plus one shared rotated key)."""
+    kind: str
+    heads: int
+    dim: int
+    vdim: int
+    kv_heads: int = 0
+    window: int = 0
+    scale: float = 1.0
+    rot_dim: int = 0          # latent attention: rotated query/key dims per head
+    kv_rank: int = 0          # latent attention: width of the cached latent
+    rot_dims: int = 0         # how many of the rot_dim dims actually rotate
+    rot_base: float = 10000.0
+    ff: int = 0
+
+    @property
+    def has_state(self) -> bool:
+        return self.kind == "hgrn2"
+
+
+@dataclass(frozen=True)
 class ModelConfig:
     name: str
-    arch: str                 # "llama" (llama / mixtral family) or "gpt2"
+    arch: str                 # "llama" (llama / mixtral family), "gpt2" or "buborax" (hybrid)
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -35,6 +62,35 @@ class ModelConfig:
     # HF ``rope_scaling`` as sorted (key, value) pairs: () = none; rope_type "llama3"
     # (Llama-3.1 / 3.2 checkpoints: low-frequency inv_freq rescaled) or "linear"
     rope_scaling: tuple = ()
+    # hybrid designs (arch "buborax"): the layer list, the shared-weight loop
+    # (start, stop, times) or (), grouped-norm group count and the residual multiplier
+    layer_specs: tuple = ()
+    loop: tuple = ()
+    norm_groups: int = 1
+    residual_mult: float = 1.0
+
+    @property
+    def is_hybrid(self) -> bool:
+        return bool(self.layer_specs)
+
+    def layer_runs(self) -> list:
+        """Execution order of a hybrid design: (layer index, pass number or -1, first of its
+        pass). Layers [start, stop) of ``loop`` run ``times`` times in a row; each run owns a
+        cache or state of its own."""
+        n = len(self.layer_specs)
+        if not self.loop:
+            return [(i, -1, False) for i in range(n)]
+        start, stop, times = self.loop
+        runs = [(i, -1, False) for i in range(start)]
+        for t in range(times):
+            runs += [(i, t, i == start) for i in range(start, stop)]
+        return runs + [(i, -1, False) for i in range(stop, n)]
+
+    @property
+    def has_state(self) -> bool:
+        """True when some layer keeps a recurrent state per sequence (state slots; such a
+        model's prefix cannot be taken from cached KV blocks alone)."""
+        return any(s.has_state for s in self.layer_specs)
 
     @property
     def is_moe(self) -> bool:
@@ -54,6 +110,12 @@ class ModelConfig:
 
     def layer_param_count(self) -> int:
         d, f = self.hidden_size, self.intermediate_size
+        if self.is_hybrid:
+            from .weights import hybrid_layer_shapes
+            import math
+            tot = sum(math.prod(s) for i in range(len(self.layer_specs))
+                      for s in hybrid_layer_shapes(self, i).values())
+            return tot // max(1, len(self.layer_specs))
         if self.arch == "gpt2":
             # c_attn (d x 3d + 3d), c_proj (d x d + d), c_fc (d x f + f), mlp c_proj (f x d + d), 2 LN
             return d * 3 * d + 3 * d + d * d + d + d * f + f + f * d + d + 4 * d
@@ -81,7 +143,18 @@ class ModelConfig:
                 + self.head_param_count())
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        if self.is_hybrid:
+            return sum(self.cache_row_width(i) for i, _, _ in self.layer_runs()) * dtype_bytes
         return 2 * self.num_layers * self.kv_size * dtype_bytes
+
+    def cache_row_width(self, layer: int) -> int:
+        """Cached elements per token of one run of hybrid layer ``layer``."""
+        s = self.layer_specs[layer]
+        if s.kind == "attention":
+            return 2 * s.kv_heads * s.dim           # normed keys + raw keys (the values)
+        if s.kind == "latent_attention":
+            return s.kv_rank + s.rot_dim
+        return 0
 
     def to_dict(self) -> dict:
         return asdict(self)
@@ -90,6 +163,11 @@ class ModelConfig:
     def from_dict(cls, d: dict) -> "ModelConfig":
         fields = cls.__dataclass_fields__.keys()
         kw = {k: v for k, v in d.items() if k in fields}
+        if kw.get("layer_specs"):
+            kw["layer_specs"] = tuple(s if isinstance(s, LayerSpec) else LayerSpec(**s)
+                                      for s in kw["layer_specs"])
+        if "loop" in kw:
+            kw["loop"] = tuple(kw["loop"] or ())
         if "rope_scaling" in kw:         # JSON turned the pairs into lists
             kw["rope_scaling"] = tuple(tuple(p) for p in (kw["rope_scaling"] or ()))
         return cls(**kw)
@@ -137,9 +215,36 @@ GPT2_TINY = replace(GPT2, name="gpt2-tiny", hidden_size=256, num_layers=2, num_h
                     num_kv_heads=4, head_dim=64, intermediate_size=1024, vocab_size=1024,
                     max_position=256, bos_token_id=1023, eos_token_id=1023)
 
+def hybrid_config(name: str, width: int, vocab: int, layer_specs, loop=(), norm_groups: int = 1,
+                  norm_eps: float = 1e-6, residual_mult: float = 1.0) -> ModelConfig:
+    """A hybrid (layer-list) ModelConfig; the llama-shaped fields hold the widest layer's sizes
+    (they only feed capacity estimates)."""
+    specs = tuple(layer_specs)
+    heads = max(s.heads for s in specs)
+    return ModelConfig(
+        name=name, arch="buborax", hidden_size=width, num_layers=len(specs), num_heads=heads,
+        num_kv_heads=max(max(s.kv_heads, 1) for s in specs), head_dim=max(s.dim for s in specs),
+        intermediate_size=max(s.ff for s in specs), vocab_size=vocab, max_position=1 << 20,
+        rope_theta=0.0, norm_eps=norm_eps, bos_token_id=0, eos_token_id=-1,
+        layer_specs=specs, loop=tuple(loop), norm_groups=norm_groups,
+        residual_mult=residual_mult)
+
+
+# Buborax at test size: every mixer kind, a loop over two layers, grouped norm, GQA in the
+# attention layer, a layer without feed-forward
+BUBORAX_TINY = hybrid_config(
+    "buborax-tiny", width=128, vocab=384,
+    layer_specs=(
+        LayerSpec("attention", heads=4, kv_heads=2, dim=32, vdim=32, window=24, scale=0.2, ff=192),
+        LayerSpec("hgrn2", heads=2, dim=32, vdim=48, ff=192),
+        LayerSpec("latent_attention", heads=4, dim=32, vdim=24, window=40, scale=0.15,
+                  rot_dim=16, kv_rank=48, rot_dims=8, rot_base=5000.0, ff=0),
+        LayerSpec("hgrn2", heads=4, dim=16, vdim=32, ff=160)),
+    loop=(1, 3, 2), norm_groups=2, norm_eps=1e-6, residual_mult=0.8)
+
 _REGISTRY = {c.name: c for c in
              (GPT2, LLAMA3_8B, LLAMA3_70B, MIXTRAL_8X7B, LLAMA_TINY, LLAMA_TINY128,
-              LLAMA_TINY8, MIXTRAL_TINY, MIXTRAL_TINY8E, GPT2_TINY)}
+              LLAMA_TINY8, MIXTRAL_TINY, MIXTRAL_TINY8E, GPT2_TINY, BUBORAX_TINY)}
 
 _ALIASES = {
     "openai-community/gpt2": "gpt2",

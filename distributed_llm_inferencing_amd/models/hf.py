@@ -25,7 +25,7 @@ from typing import Dict, Iterable, Iterator, Optional, Tuple
 import torch
 
 from .configs import ModelConfig
-from .weights import from_hf_state_dict
+from .weights import from_buborax_state_dict, from_hf_state_dict
 
 
 def is_hf_dir(d) -> bool:
@@ -37,7 +37,7 @@ def is_hf_dir(d) -> bool:
         c = json.loads(cj.read_text())
     except (OSError, ValueError):
         return False
-    return "model_type" in c and ((d / "model.safetensors").exists()
+    return ("model_type" in c or c.get("architecture") in NATIVE_ARCHS) and ((d / "model.safetensors").exists()
                                   or (d / "model.safetensors.index.json").exists())
 
 
@@ -58,8 +58,58 @@ def find_hf_dir(root: str, name: str) -> Optional[Path]:
     return None
 
 
+NATIVE_ARCHS = ("Buborax",)
+
+
+def buborax_config(c: dict, name: Optional[str] = None) -> ModelConfig:
+    """A Buborax ``config.json``: ``width``, ``vocab``, ``norm`` {eps, groups},
+    ``residual_mult``, ``loop`` {start, stop, times} (optional) and ``layers``, a list of
+    {type, mixer {...}, mlp {kind, ff} or null}. Every size and constant is read from it."""
+    from .configs import LayerSpec, hybrid_config
+    specs = []
+    for L in c["layers"]:
+        mx, kind = L["mixer"], L["type"]
+        mlp = L.get("mlp")
+        if mlp and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"unsupported feed-forward kind '{mlp.get('kind')}'")
+        ff = int(mlp["ff"]) if mlp else 0
+        H, d = int(mx["heads"]), int(mx["dim"])
+        if kind == "attention":
+            G = int(mx.get("kv_heads") or H)
+            dv = int(mx.get("vdim", d))
+            if dv != d or H % G:
+                raise ValueError("attention: the values are the keys (vdim == dim) and heads "
+                                 "must be a multiple of kv_heads")
+            specs.append(LayerSpec("attention", heads=H, kv_heads=G, dim=d, vdim=dv,
+                                   window=int(mx["mask"]["size"]), scale=float(mx["scale"]),
+                                   ff=ff))
+        elif kind == "hgrn2":
+            specs.append(LayerSpec("hgrn2", heads=H, dim=d, vdim=int(mx["vdim"]), ff=ff))
+        elif kind == "latent_attention":
+            rot = mx.get("rot") or {}
+            dr = int(mx["rot_dim"])
+            specs.append(LayerSpec("latent_attention", heads=H, kv_heads=1, dim=d,
+                                   vdim=int(mx["vdim"]), window=int(mx["mask"]["size"]),
+                                   scale=float(mx["scale"]), rot_dim=dr,
+                                   kv_rank=int(mx["kv_rank"]), rot_dims=int(rot.get("dims", dr)),
+                                   rot_base=float(rot.get("base", 10000.0)), ff=ff))
+        else:
+            raise ValueError(f"unsupported mixer type '{kind}'")
+    lp = c.get("loop")
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else ()
+    if loop and not (0 <= loop[0] < loop[1] <= len(specs) and loop[2] >= 1):
+        raise ValueError(f"bad loop {loop} for {len(specs)} layers")
+    norm = c.get("norm") or {}
+    return hybrid_config(name or c.get("_name_or_path") or "buborax", int(c["width"]),
+                         int(c["vocab"]), specs, loop, int(norm.get("groups", 1)),
+                         float(norm.get("eps", 1e-6)), float(c.get("residual_mult", 1.0)))
+
+
 def config_from_hf(c: dict, name: Optional[str] = None) -> ModelConfig:
-    """Map a HF ``config.json`` (llama / mistral / mixtral / gpt2 model types)."""
+    """Map a ``config.json``: HF llama / mistral / mixtral / gpt2 model types, or one of the
+    native layer-list designs (``architecture``: Buborax)."""
+    if c.get("architecture") == "Buborax":
+        return buborax_config(c, name)
     mt = c.get("model_type", "")
     name = name or c.get("_name_or_path") or mt
     if mt == "gpt2":
@@ -169,7 +219,11 @@ def load_hf_dir(d, device="cpu", dtype=torch.bfloat16, name: Optional[str] = Non
     cfg = config_from_hf(json.loads((d / "config.json").read_text()), name)
     sd = LazyStateDict(d)
     try:
-        params = from_hf_state_dict(cfg, sd, layers=layers, first=first, last=last, dtype=dtype)
+        if cfg.is_hybrid:
+            params = from_buborax_state_dict(cfg, sd, dtype=dtype)
+        else:
+            params = from_hf_state_dict(cfg, sd, layers=layers, first=first, last=last,
+                                        dtype=dtype)
     finally:
         sd.close()
     dev = torch.device(device)

@@ -1,0 +1,149 @@
+"""Hybrid decoder (arch ``buborax``): a layer list that mixes windowed attention, latent
+attention and a gated linear recurrence, with a shared-weight loop, grouped RMS norms and an
+fp32 residual stream — served by the same engine, scheduler, block manager and runner as the
+transformer families.
+
+    embed (fp32) -> per layer run: x += m * mixer(gnorm(x)); x += m * ff(gnorm(x))
+                 -> gnorm -> LM head (fp32 logits) -> sampler
+
+* Layers [start, stop) of the loop run ``times`` times with the same weights; a pass starts
+  with x = W_in [x ; x0] + step[pass] (x0 = the embedding output). Every run owns its cache or
+  state (``engine.kv_cache.HybridCache``).
+* The residual stream and every norm are fp32; GEMM operands use the storage dtype of the
+  weights (bf16 when serving; fp32 weights give an all-fp32 model). Each residual add is fused
+  with the norm that follows it (``ops.hybrid.resadd_groupnorm``).
+* Every step kind — whole prompts, prompt portions, decode rows, mixed — runs the same path:
+  new tokens are written to the paged caches, then attend through the block tables, so a
+  position's logits do not depend on how its sequence was cut into steps.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..engine.batch import DeviceBatch
+from ..ops import hybrid as H
+from .configs import ModelConfig
+from .mixers import MIXERS, StepView, derive_constants
+from .model import TransformerLM
+
+
+class HybridLM(TransformerLM):
+    # the scheduler builds block tables for every step, not only chunked ones
+    needs_block_tables = True
+
+    def __init__(self, cfg: ModelConfig, params: Dict[str, torch.Tensor], layer_start: int = 0,
+                 layer_end: Optional[int] = None, device="cpu", expert_range=None):
+        if layer_start != 0 or (layer_end is not None and layer_end != cfg.num_layers):
+            raise ValueError("hybrid designs run on one stage (the loop entry reads the "
+                             "embedding output)")
+        super().__init__(cfg, params, 0, None, device)
+        self.dtype = params["embed"].dtype
+        self.runs = cfg.layer_runs()
+        for spec, lp in zip(cfg.layer_specs, self.layers):
+            derive_constants(spec, lp, self.device)
+        self._cu: Dict[int, torch.Tensor] = {}
+        # debugging aid: when a list, forward_layers appends the residual after every run
+        self.layer_trace: Optional[List[torch.Tensor]] = None
+
+    def to(self, device):
+        super().to(device)
+        for spec, lp in zip(self.cfg.layer_specs, self.layers):
+            derive_constants(spec, lp, self.device)
+        self._cu.clear()
+        return self
+
+    # ------------------------------------------------------------------ step metadata
+    def _step_view(self, b: DeviceBatch, block_size: int) -> StepView:
+        if b.is_prefill:
+            cu, mx = b.cu_seqlens, b.max_seqlen
+        else:                                   # decode: one row per sequence
+            n = b.num_tokens
+            cu = self._cu.get(n)
+            if cu is None:
+                cu = self._cu[n] = torch.arange(n + 1, dtype=torch.int32, device=self.device)
+            mx = 1
+        if b.block_tables is None:
+            raise ValueError("hybrid models attend through the paged cache: the step carries "
+                             "no block tables")
+        return StepView(cu, mx, b.positions, b.slot_mapping, b.block_tables, block_size,
+                        b.state_slots)
+
+    # ------------------------------------------------------------------ forward
+    def embed(self, b: DeviceBatch) -> torch.Tensor:
+        return H.embedding_f32(b.input_ids, self.params["embed"])[0]
+
+    def forward_layers(self, x: torch.Tensor, b: DeviceBatch, kv_caches) -> torch.Tensor:
+        cfg, p = self.cfg, self.params
+        eps, groups, m = cfg.norm_eps, cfg.norm_groups, cfg.residual_mult
+        step = self._step_view(b, kv_caches.block_size)
+        entries = kv_caches.entries
+        x0 = x.clone() if cfg.loop else None
+        pending = None                      # a sub-block's fp32 output awaiting its add
+        for ri, (li, t, first) in enumerate(self.runs):
+            spec, lp = cfg.layer_specs[li], self.layers[li]
+            if first:
+                if pending is not None:
+                    H.resadd_groupnorm(x, pending, None, groups, eps, mult=m)
+                    pending = None
+                y = H.linear_any(H.concat_cast(x, x0, self.dtype), p["loop_in"])
+                h = H.resadd_groupnorm(x, y, lp["norm1"], groups, eps, mult=1.0, keep=0.0,
+                                       bias=p["loop_step"][t])
+            else:
+                h = H.resadd_groupnorm(x, pending, lp["norm1"], groups, eps, mult=m)
+            y = MIXERS[spec.kind](spec, lp, h, step, entries[ri], eps)
+            if spec.ff:
+                h = H.resadd_groupnorm(x, y, lp["norm2"], groups, eps, mult=m)
+                act = H.gelu_mul(H.linear_any(h, lp["w_gu"]), spec.ff, self.dtype)
+                y = H.linear_any(act, lp["w_down"])
+            pending = y
+            if self.layer_trace is not None:
+                H.resadd_groupnorm(x, pending, None, groups, eps, mult=m)
+                pending = None
+                self.layer_trace.append(x.clone())
+        if pending is not None:
+            H.resadd_groupnorm(x, pending, None, groups, eps, mult=m)
+        return x
+
+    def final_hidden(self, hidden: torch.Tensor, b: DeviceBatch) -> torch.Tensor:
+        cfg, p = self.cfg, self.params
+        if b.logit_rows is not None:
+            rows = b.logit_rows
+        elif b.is_prefill:
+            rows = b.last_token_idx
+        else:
+            return H.resadd_groupnorm(hidden, None, p["final_norm"], cfg.norm_groups,
+                                      cfg.norm_eps)
+        return H.groupnorm_rows(hidden, rows, p["final_norm"], cfg.norm_groups, cfg.norm_eps)
+
+    def head_logits(self, h: torch.Tensor) -> torch.Tensor:
+        return H.linear_any(h, self.params["lm_head"], out_f32=True)
+
+    def forward(self, b: DeviceBatch, kv_caches, hidden: Optional[torch.Tensor] = None,
+                return_logits: bool = False):
+        """Sampled int32 tokens [S] (and the logits when asked). With ``b.logit_rows`` the
+        logits of exactly those rows are returned and nothing is sampled."""
+        x = self.forward_layers(self.embed(b), b, kv_caches)
+        lg = self.logits(x, b)
+        if b.logit_rows is not None:
+            return lg
+        tok = self.sample(lg, b)
+        return (tok, lg) if return_logits else tok
+
+    # ------------------------------------------------------------------ planning
+    def gemm_shapes(self, M: int):
+        """(shapes, weights) of the projection GEMMs a step of M rows runs on the tuned tile
+        family (fp32-output plans; other shapes run the shape-agnostic kernel)."""
+        shapes, weights = [], {}
+        if self.dtype != torch.bfloat16:
+            return shapes, weights
+        mats = [w for lp in self.layers for w in lp.values()
+                if isinstance(w, torch.Tensor) and w.dim() == 2 and w.dtype == self.dtype]
+        mats += [self.params[k] for k in ("loop_in", "lm_head") if k in self.params]
+        for w in mats:
+            n, k = w.shape
+            if k % 64 == 0 and (n, k) not in weights and n >= 16:
+                shapes.append((M, n, k, "f32"))
+                weights[(n, k)] = w
+        return shapes, weights

@@ -240,7 +240,9 @@ class TransformerLM:
     def final_hidden(self, hidden: torch.Tensor, b: DeviceBatch) -> torch.Tensor:
         """Final norm of the last token of each sequence -> bf16 [S, D]."""
         cfg, p = self.cfg, self.params
-        if b.is_prefill:
+        if b.logit_rows is not None:
+            hidden = hidden.index_select(0, b.logit_rows)
+        elif b.is_prefill:
             hidden = hidden.index_select(0, b.last_token_idx)
         if cfg.arch == "gpt2":
             return ops.layernorm(hidden, p["final_norm"], p["final_norm_b"], cfg.norm_eps)
@@ -277,5 +279,7 @@ class TransformerLM:
         if self.vocab_parallel:          # the LM head runs sliced on every pipeline rank
             return self.final_hidden(x, b)
         lg = self.logits(x, b)
+        if b.logit_rows is not None:     # scoring / trace replay: these rows' logits, no sampling
+            return lg
         tok = self.sample(lg, b)
         return (tok, lg) if return_logits else tok

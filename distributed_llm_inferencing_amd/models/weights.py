@@ -27,7 +27,42 @@ from ..ops.reference import interleave_gate_up
 INIT_STD = 0.02
 
 
+def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
+    """In-memory tensors of hybrid layer ``i`` (``layers.{i}.``), projections that read the
+    same input fused row-wise:
+      attention:        w_in [(H + G + H)*d, D] = q | k | gate, q_norm [d], k_norm [d],
+                        talk [H, H] fp32, wo [D, H*d]
+      hgrn2:            w_in [(2*H*d + H*dv), D] = q | f | v, f_b [H*d], lower [H*d],
+                        o_norm [dv], wo [D, H*dv]
+      latent_attention: w_in [H*(d+dr) + r + dr, D] = q | compressed kv, c_norm [r],
+                        w_ukT [H, r, d] (per head, transposed: the absorb projection),
+                        w_uv [H, dv, r], wo [D, H*dv]
+      feed-forward:     norm2 [D], w_gu [2F, D] = gate | up, w_down [D, F]"""
+    D = cfg.hidden_size
+    s = cfg.layer_specs[i]
+    p = f"layers.{i}."
+    H, d, dv = s.heads, s.dim, s.vdim
+    out = {p + "norm1": (D,)}
+    if s.kind == "attention":
+        out.update({p + "w_in": ((2 * H + s.kv_heads) * d, D), p + "q_norm": (d,),
+                    p + "k_norm": (d,), p + "talk": (H, H), p + "wo": (D, H * d)})
+    elif s.kind == "hgrn2":
+        out.update({p + "w_in": (2 * H * d + H * dv, D), p + "f_b": (H * d,),
+                    p + "lower": (H * d,), p + "o_norm": (dv,), p + "wo": (D, H * dv)})
+    elif s.kind == "latent_attention":
+        out.update({p + "w_in": (H * (d + s.rot_dim) + s.kv_rank + s.rot_dim, D),
+                    p + "c_norm": (s.kv_rank,), p + "w_ukT": (H, s.kv_rank, d),
+                    p + "w_uv": (H, dv, s.kv_rank), p + "wo": (D, H * dv)})
+    else:
+        raise ValueError(f"unknown mixer kind '{s.kind}'")
+    if s.ff:
+        out.update({p + "norm2": (D,), p + "w_gu": (2 * s.ff, D), p + "w_down": (D, s.ff)})
+    return out
+
+
 def layer_param_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
+    if cfg.is_hybrid:
+        return hybrid_layer_shapes(cfg, i)
     d, f, hd = cfg.hidden_size, cfg.intermediate_size, cfg.head_dim
     p = f"layers.{i}."
     if cfg.arch == "gpt2":
@@ -47,6 +82,13 @@ def layer_param_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
 def global_param_shapes(cfg: ModelConfig, first: bool, last: bool) -> Dict[str, tuple]:
     d, v = cfg.hidden_size, cfg.vocab_size
     s: Dict[str, tuple] = {}
+    if cfg.is_hybrid:
+        # the loop entry re-reads the embedding output, so a stage that runs loop layers
+        # holds the embedding too (hybrid designs run on one stage)
+        s.update({"embed": (v, d), "final_norm": (d,), "lm_head": (v, d)})
+        if cfg.loop:
+            s.update({"loop_in": (d, 2 * d), "loop_step": (cfg.loop[2], d)})
+        return s
     if first or (last and cfg.tie_embeddings):
         s["embed"] = (v, d)
     if first and cfg.arch == "gpt2":
@@ -75,7 +117,8 @@ def stage_param_shapes(cfg: ModelConfig, layer_start: int, layer_end: int, first
 
 
 def _is_norm_weight(name: str) -> bool:
-    return name.endswith(("attn_norm", "mlp_norm", "final_norm", "ln1_w", "ln2_w"))
+    return name.endswith(("attn_norm", "mlp_norm", "final_norm", "ln1_w", "ln2_w", "norm1",
+                          "norm2", "q_norm", "k_norm", "c_norm", "o_norm"))
 
 
 def _is_bias(name: str) -> bool:
@@ -88,9 +131,12 @@ def random_init(shapes: Dict[str, tuple], device, dtype=torch.bfloat16, seed: in
     pipeline stage generates exactly the slice the full model would hold."""
     out = {}
     dev = torch.device(device)
+    hybrid = any(n.endswith(".norm1") for n in shapes)
     for name in sorted(shapes):
         shape = shapes[name]
-        if _is_norm_weight(name):
+        if hybrid and not _is_norm_weight(name):
+            out[name] = _hybrid_init(name, shape, dev, dtype, seed)
+        elif _is_norm_weight(name):
             out[name] = torch.ones(shape, dtype=dtype, device=dev)
         elif _is_bias(name):
             out[name] = torch.zeros(shape, dtype=dtype, device=dev)
@@ -101,6 +147,23 @@ def random_init(shapes: Dict[str, tuple], device, dtype=torch.bfloat16, seed: in
             t.normal_(0.0, std, generator=g)
             out[name] = t
     return out
+
+
+def _hybrid_init(name: str, shape: tuple, dev, dtype, seed: int) -> torch.Tensor:
+    """Random values for the hybrid family's tensors that a plain normal(0, 0.02) would make
+    degenerate: head-mixing matrices near the identity (fp32), forget-gate lower bounds in
+    [0, 0.9), gate biases and loop step vectors of unit-ish size, and input projections scaled
+    like 1/sqrt(fan_in) so that normed queries, gates and recurrences see O(1) inputs."""
+    g = torch.Generator(device="cpu")
+    g.manual_seed((seed * 1_000_003 + _name_hash(name)) & 0x7FFF_FFFF_FFFF)
+    if name.endswith(".talk"):
+        t = torch.eye(shape[0]) + 0.2 * torch.randn(shape, generator=g)
+        return t.to(dev, torch.float32)
+    if name.endswith(".lower"):
+        return (0.9 * torch.rand(shape, generator=g)).to(dev, dtype)
+    if name.endswith((".f_b", "loop_step")):
+        return (0.5 * torch.randn(shape, generator=g)).to(dev, dtype)
+    return (torch.randn(shape, generator=g) / shape[-1] ** 0.5).to(dev, dtype)
 
 
 def slice_experts(name: str, t: torch.Tensor, expert_range: Optional[tuple]) -> torch.Tensor:
@@ -202,4 +265,41 @@ def from_hf_state_dict(cfg: ModelConfig, sd: Dict[str, torch.Tensor],
             out[p + "w_gu"] = cv(interleave_gate_up(sd[h + "mlp.gate_proj.weight"],
                                                     sd[h + "mlp.up_proj.weight"]))
             out[p + "w_down"] = cv(sd[h + "mlp.down_proj.weight"])
+    return out
+
+
+# ----------------------------------------------------------------------------- Buborax files
+def from_buborax_state_dict(cfg: ModelConfig, sd, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Convert a Buborax checkpoint (tensor names ``embed``, ``head``, ``final.norm``,
+    ``loop.in``, ``loop.step``, ``l<i>.norm1|norm2``, ``l<i>.mix.*``, ``l<i>.mlp.*``; linear
+    weights [out, in]) into the in-memory layout of ``hybrid_layer_shapes``."""
+    cv = lambda t: t.detach().to(dtype).contiguous()  # noqa: E731
+    out = {"embed": cv(sd["embed"]), "lm_head": cv(sd["head"]), "final_norm": cv(sd["final.norm"])}
+    if cfg.loop:
+        out["loop_in"] = cv(sd["loop.in"])
+        out["loop_step"] = cv(sd["loop.step"])
+    for i, s in enumerate(cfg.layer_specs):
+        a, p = f"l{i}.", f"layers.{i}."
+        m = a + "mix."
+        out[p + "norm1"] = cv(sd[a + "norm1"])
+        H, d, dv = s.heads, s.dim, s.vdim
+        if s.kind == "attention":
+            out[p + "w_in"] = cv(torch.cat([sd[m + "q"], sd[m + "k"], sd[m + "g"]], 0))
+            out[p + "q_norm"], out[p + "k_norm"] = cv(sd[m + "q.norm"]), cv(sd[m + "k.norm"])
+            out[p + "talk"] = sd[m + "talk"].detach().float().contiguous()
+        elif s.kind == "hgrn2":
+            out[p + "w_in"] = cv(torch.cat([sd[m + "q"], sd[m + "f"], sd[m + "v"]], 0))
+            out[p + "f_b"], out[p + "lower"] = cv(sd[m + "f.b"]), cv(sd[m + "lower"])
+            out[p + "o_norm"] = cv(sd[m + "norm"])
+        else:
+            out[p + "w_in"] = cv(torch.cat([sd[m + "q"], sd[m + "dkv"]], 0))
+            out[p + "c_norm"] = cv(sd[m + "dkv.norm"])
+            uk = sd[m + "uk"].detach().reshape(H, d, s.kv_rank)
+            out[p + "w_ukT"] = cv(uk.transpose(1, 2))
+            out[p + "w_uv"] = cv(sd[m + "uv"].detach().reshape(H, dv, s.kv_rank))
+        out[p + "wo"] = cv(sd[m + "o"])
+        if s.ff:
+            out[p + "norm2"] = cv(sd[a + "norm2"])
+            out[p + "w_gu"] = cv(torch.cat([sd[a + "mlp.gate"], sd[a + "mlp.up"]], 0))
+            out[p + "w_down"] = cv(sd[a + "mlp.down"])
     return out

@@ -1,0 +1,213 @@
+"""Ops of the hybrid model family (models/hybrid.py): fp32 residual stream and norms, grouped
+RMS norm, windowed attention with distance bias / head mixing / output gate over token-major
+paged caches, latent (compressed-kv) attention in the absorbed form, a gated linear recurrence
+with per-sequence state slots, and a shape-agnostic GEMM.
+
+Dispatch is the package's: CUDA (HIP) tensors run the gfx950 kernels (``csrc/kernels``:
+hybrid_elementwise.hip, window_attention.hip, recurrent.hip, gemm_any.hip), CPU tensors the
+PyTorch reference (``ops/reference.py``). The storage dtype (bf16 when serving, fp32 in the
+exact mode) is the dtype of the weights; kernels take it as ``dt``.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _native as N
+from . import gemm as G
+from . import reference as R
+
+_call = N.call
+_p = N.ptr
+
+
+def _dt(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return 0
+    if dtype == torch.float32:
+        return 1
+    raise ValueError(f"hybrid ops: storage dtype {dtype} (bfloat16 or float32)")
+
+
+def _st():
+    return N.stream_ptr()
+
+
+# ----------------------------------------------------------------------------- GEMM
+def linear_any(x: torch.Tensor, w: torch.Tensor, out_f32: bool = True,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [M, K] @ w [N, K]^T with fp32 accumulation -> fp32 (or the storage dtype). bf16 shapes
+    the tuned tile family accepts (K a multiple of its K-tile, 16-byte rows) run there; every
+    other shape, and fp32 operands, run the shape-agnostic kernel."""
+    if not x.is_cuda:
+        y = R.linear(x, w, out_dtype=torch.float32 if out_f32 else x.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+    M, K = x.shape
+    Nn = w.shape[0]
+    if x.dtype != w.dtype or w.shape[1] != K or x.stride(1) != 1 or w.stride(1) != 1:
+        raise ValueError("linear_any: operand dtypes / inner dims do not match")
+    f32 = out_f32 or x.dtype == torch.float32
+    if out is None:
+        out = torch.empty(M, Nn, dtype=torch.float32 if f32 else x.dtype, device=x.device)
+    if (x.dtype == torch.bfloat16 and K % 64 == 0 and x.stride(0) % 8 == 0
+            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and out.stride(1) == 1):
+        from . import _gemm_native
+        return _gemm_native(x, w, "f32" if f32 else "none", out=out)
+    _call("dli_gemm_any", _p(x), x.stride(0), _p(w), w.stride(0), _p(out), out.stride(0), M, Nn,
+          K, _dt(x.dtype), int(f32), 1, 0, 0, 0, _st())
+    return out
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """Per-head projection: out[:, h, :n] = x[:, h, :] @ w[h]^T for x [T, H, k], w [H, n, k],
+    out [T, H, >= n] (the result lands in the first n columns of each head's row; x and out may
+    be column slices of wider rows). One batched launch."""
+    T, H, k = x.shape
+    n = w.shape[1]
+    if not x.is_cuda:
+        y = torch.einsum("thk,hnk->thn", x.float(), w.float())
+        out[:, :, :n] = y.to(out.dtype)
+        return out
+    if x.stride(2) != 1 or w.stride(2) != 1 or out.stride(2) != 1 or x.dtype != w.dtype:
+        raise ValueError("head_linear: inner dims must be contiguous")
+    _call("dli_gemm_any", _p(x), x.stride(0), _p(w), w.stride(1), _p(out), out.stride(0), T, n, k,
+          _dt(x.dtype), int(out.dtype == torch.float32), H, x.stride(1), w.stride(0),
+          out.stride(1), _st())
+    return out
+
+
+# ----------------------------------------------------------------------------- rows
+def embedding_f32(ids: torch.Tensor, table: torch.Tensor, copy: bool = False):
+    """fp32 rows of ``table`` (and a second copy when asked: the loop input)."""
+    if not table.is_cuda:
+        x = table[ids.long()].float()
+        return (x, x.clone()) if copy else (x, None)
+    T, D = ids.shape[0], table.shape[1]
+    x = torch.empty(T, D, dtype=torch.float32, device=table.device)
+    x0 = torch.empty_like(x) if copy else None
+    _call("dli_embedding_f32", _p(x), _p(x0), _p(ids), _p(table), T, D, table.shape[0],
+          _dt(table.dtype), _st())
+    return x, x0
+
+
+def resadd_groupnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[torch.Tensor],
+                     groups: int, eps: float, mult: float = 1.0, keep: float = 1.0,
+                     bias: Optional[torch.Tensor] = None, dtype=None) -> Optional[torch.Tensor]:
+    """In place on the fp32 stream: x = keep * x + mult * y + bias (y, bias optional); returns
+    the grouped RMS norm of the new x times ``w`` in the storage dtype (None when w is None)."""
+    dtype = dtype or (w.dtype if w is not None else torch.bfloat16)
+    if not x.is_cuda:
+        if keep != 1.0:
+            x.mul_(keep) if keep != 0.0 else x.zero_()
+        if y is not None:
+            x.add_(y.float(), alpha=mult)
+        if bias is not None:
+            x.add_(bias.float())
+        return None if w is None else R.group_rmsnorm(x, w, groups, eps, dtype)
+    rows, dim = x.shape
+    h = torch.empty(rows, dim, dtype=dtype, device=x.device) if w is not None else None
+    _call("dli_resadd_groupnorm", _p(x), _p(y), y.stride(0) if y is not None else 0, _p(bias),
+          float(keep), float(mult), _p(w), _p(h), dim, rows, dim, groups, float(eps), None,
+          _dt(dtype), _st())
+    return h
+
+
+def groupnorm_rows(x: torch.Tensor, rows_idx: torch.Tensor, w: torch.Tensor, groups: int,
+                   eps: float) -> torch.Tensor:
+    """Grouped RMS norm of the rows ``rows_idx`` (int64) of the fp32 stream."""
+    if not x.is_cuda:
+        return R.group_rmsnorm(x.index_select(0, rows_idx), w, groups, eps, w.dtype)
+    n, dim = rows_idx.shape[0], x.shape[1]
+    h = torch.empty(n, dim, dtype=w.dtype, device=x.device)
+    _call("dli_resadd_groupnorm", _p(x), None, 0, None, 1.0, 1.0, _p(w), _p(h), dim, n, dim,
+          groups, float(eps), _p(rows_idx), _dt(w.dtype), _st())
+    return h
+
+
+def concat_cast(a: torch.Tensor, b: torch.Tensor, dtype) -> torch.Tensor:
+    """[a ; b] (fp32 [T, D] each) as [T, 2D] in the storage dtype."""
+    if not a.is_cuda:
+        return torch.cat([a, b], 1).to(dtype)
+    T, D = a.shape
+    out = torch.empty(T, 2 * D, dtype=dtype, device=a.device)
+    _call("dli_concat_cast", _p(out), _p(a), _p(b), T, D, _dt(dtype), _st())
+    return out
+
+
+def gelu_mul(gu: torch.Tensor, F_: int, dtype) -> torch.Tensor:
+    """gelu_tanh(gu[:, :F]) * gu[:, F:2F] for an fp32 [T, 2F] projection."""
+    if not gu.is_cuda:
+        return R.gelu_mul(gu, F_, dtype)
+    T = gu.shape[0]
+    out = torch.empty(T, F_, dtype=dtype, device=gu.device)
+    _call("dli_gelu_mul", _p(out), F_, _p(gu), gu.stride(0), T, F_, _dt(dtype), _st())
+    return out
+
+
+# ----------------------------------------------------------------------------- mixers
+def attn_prepare(proj, qw, kw, eps, H, G, d, kcache, vcache, slots):
+    dtype = qw.dtype
+    if not proj.is_cuda:
+        return R.attn_prepare(proj, qw, kw, eps, H, G, d, kcache, vcache, slots, dtype)
+    T = proj.shape[0]
+    q = torch.empty(T, H * d, dtype=dtype, device=proj.device)
+    _call("dli_attn_prepare", _p(proj), proj.stride(0), _p(qw), _p(kw), float(eps), T, H, G, d,
+          _p(q), _p(kcache), _p(vcache), _p(slots), _dt(dtype), _st())
+    return q
+
+
+def mla_prepare(proj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots, cache):
+    """Returns (q_nope [T, H, d], q_full [T, H, r + dr]) with q_full's rotated tail written;
+    its first r columns are for the absorb projection (``head_linear``)."""
+    dtype = cw.dtype
+    T = proj.shape[0]
+    if not proj.is_cuda:
+        qn, qr = R.mla_prepare(proj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots,
+                               cache, dtype)
+        qf = torch.zeros(T, H, r + dr, dtype=dtype)
+        qf[:, :, r:] = qr
+        return qn, qf
+    qn = torch.empty(T, H, d, dtype=dtype, device=proj.device)
+    qf = torch.empty(T, H, r + dr, dtype=dtype, device=proj.device)
+    _call("dli_mla_prepare", _p(proj), proj.stride(0), _p(cw), float(eps), T, H, d, dr, r,
+          rot_dims, _p(inv_freq), _p(positions), _p(slots), _p(qn), _p(qf), _p(cache),
+          _dt(dtype), _st())
+    return qn, qf
+
+
+def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, positions,
+                     block_tables, block_size, window, scale, slopes=None, talk=None, gate=None):
+    """See ``reference.window_attention`` / window_attention.hip. q [T, H*dq] (storage dtype);
+    caches are token-major rows; returns [T, H*dv] in the storage dtype."""
+    if not q.is_cuda:
+        return R.window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions,
+                                  block_tables, block_size, window, scale, slopes, talk, gate,
+                                  out_dtype=q.dtype)
+    T = q.shape[0]
+    S = cu_seqlens.shape[0] - 1
+    out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    _call("dli_window_attention", _p(q), q.stride(0), _p(k_cache), k_cache.stride(0),
+          _p(v_cache), v_cache.stride(0), _p(out), out.stride(0), _p(gate),
+          gate.stride(0) if gate is not None else 0, _p(slopes), _p(talk), _p(cu_seqlens),
+          _p(positions), _p(block_tables), block_tables.stride(0), block_size, S,
+          int(max_seqlen), H, G, dq, dv, int(window), float(scale), _dt(q.dtype), _st())
+    return out
+
+
+def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, positions, H, d, dv):
+    dtype = norm_w.dtype
+    if not proj.is_cuda:
+        return R.hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, positions,
+                       H, d, dv, dtype)
+    T = proj.shape[0]
+    S = cu_seqlens.shape[0] - 1
+    out = torch.empty(T, H * dv, dtype=dtype, device=proj.device)
+    _call("dli_hgrn2", _p(proj), proj.stride(0), _p(f_bias), _p(lower), _p(norm_w), float(eps),
+          _p(state), _p(slots), _p(cu_seqlens), _p(positions), _p(out), out.stride(0), S, H, d,
+          dv, _dt(dtype), _st())
+    return out

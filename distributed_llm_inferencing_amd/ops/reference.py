@@ -376,3 +376,145 @@ def moe_mlp(x: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor,
         y = linear(h, w_down[le]).float()
         out.index_add_(0, rows, y * topk_w[rows, slot][:, None])
     return out.to(x.dtype)
+
+
+# ----------------------------------------------------------------------------- hybrid family
+# Mixed attention / recurrent designs (models/hybrid.py): fp32 residual stream and norms, GEMM
+# operands in the storage dtype. Layouts shared with the HIP kernels:
+# * token-major paged caches: row ``slot`` of ``[num_slots, width]`` (slot = block * block_size
+#   + offset), kv head g at columns ``[g*d, (g+1)*d)``
+# * recurrent state ``[state_slots, H, d, dv]`` fp32, one slot per live sequence
+def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """x fp32 [T, D] cut into ``groups`` equal parts, each divided by its own
+    sqrt(mean(part^2) + eps); the whole times w."""
+    T, D = x.shape
+    xg = x.float().reshape(T, groups, D // groups)
+    n = xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps)
+    return (n.reshape(T, D) * w.float()).to(out_dtype)
+
+
+def gelu_mul(gu: torch.Tensor, F_: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """gelu_tanh(gu[:, :F]) * gu[:, F:2F] (plain concatenation, fp32 in)."""
+    g, u = gu[:, :F_].float(), gu[:, F_:2 * F_].float()
+    return (F.gelu(g, approximate="tanh") * u).to(out_dtype)
+
+
+def attn_prepare(proj, qw, kw, eps, H, G, d, kcache, vcache, slots, out_dtype):
+    """proj fp32 [T, >= (H+G)*d] = [q | k | ...]: per-head RMS norm (shared weights) of q and k;
+    normed k -> kcache rows, raw k -> vcache rows; returns normed q [T, H*d]."""
+    T = proj.shape[0]
+    q = proj[:, :H * d].float().reshape(T, H, d)
+    k = proj[:, H * d:(H + G) * d].float().reshape(T, G, d)
+    qn = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw.float()
+    kn = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw.float()
+    ok = slots >= 0
+    idx = slots[ok].long()
+    kcache[idx] = kn.reshape(T, G * d)[ok].to(kcache.dtype)
+    vcache[idx] = k.reshape(T, G * d)[ok].to(vcache.dtype)
+    return qn.reshape(T, H * d).to(out_dtype)
+
+
+def rotate_interleaved(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
+                       rot_dims: int) -> torch.Tensor:
+    """Pairs (2i, 2i+1), i < rot_dims/2, of the last dim rotate by positions * inv_freq[i]
+    (fp32 angles); the rest passes unchanged. x [..., T, n] with T = len(positions) on dim -2
+    or x [T, n]."""
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    c, s = ang.cos(), ang.sin()
+    out = x.clone()
+    a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+    if x.dim() == 3:          # [T, H, n]
+        c, s = c[:, None, :], s[:, None, :]
+    out[..., 0:rot_dims:2] = a * c - b * s
+    out[..., 1:rot_dims:2] = b * c + a * s
+    return out
+
+
+def mla_prepare(proj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots, cache,
+                out_dtype):
+    """proj fp32 [T, H*(d+dr) + r + dr] = [q heads | compressed kv | shared rotated key].
+    Cache row = [normed latent | rotated key]. Returns (q_nope [T, H, d], q_rot [T, H, dr])."""
+    T = proj.shape[0]
+    q = proj[:, :H * (d + dr)].float().reshape(T, H, d + dr)
+    dkv = proj[:, H * (d + dr):H * (d + dr) + r + dr].float()
+    c = dkv[:, :r]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * cw.float()
+    kr = rotate_interleaved(dkv[:, r:], positions, inv_freq, rot_dims)
+    ok = slots >= 0
+    cache[slots[ok].long()] = torch.cat([c, kr], 1)[ok].to(cache.dtype)
+    qr = rotate_interleaved(q[:, :, d:], positions, inv_freq, rot_dims)
+    return q[:, :, :d].to(out_dtype).contiguous(), qr.to(out_dtype)
+
+
+def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions, block_tables,
+                     block_size, window, scale, slopes=None, talk=None, gate=None,
+                     out_dtype=None):
+    """q [T, H*dq]; k_cache rows [slots, G*dq]; v_cache rows [slots, >= G*dv] (may be k_cache:
+    values = the first dv columns of each kv head's... row when G == 1). Every query at position
+    p attends cached positions [max(0, p-window+1), p] of its sequence. fp32 softmax; ``talk``
+    [H, H] mixes the heads' normalised weights; ``slopes`` [H] subtract slope*(p-j); ``gate``
+    fp32 [T, H*dv] multiplies the output by its sigmoid."""
+    T = q.shape[0]
+    out = torch.zeros(T, H * dv, dtype=torch.float32, device=q.device)
+    cu = cu_seqlens.tolist()
+    for s in range(len(cu) - 1):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0:
+            continue
+        pos = positions[t0:t1].long()
+        ctx = int(pos.max()) + 1
+        j = torch.arange(ctx, device=q.device)
+        sl = (block_tables[s].long()[j // block_size] * block_size + j % block_size)
+        kk = k_cache[sl][:, :G * dq].float().reshape(ctx, G, dq)
+        vv = v_cache[sl].float()
+        vv = torch.stack([vv[:, g * dv:(g + 1) * dv] for g in range(G)], 1)   # [ctx, G, dv]
+        qq = q[t0:t1].float().reshape(t1 - t0, H, dq)
+        rep = H // G
+        ke = kk.repeat_interleave(rep, dim=1)                                   # [ctx, H, dq]
+        sc = torch.einsum("thd,jhd->htj", qq, ke) * scale
+        dist = (pos[:, None] - j[None, :]).float()                              # [n, ctx]
+        if slopes is not None:
+            sc = sc - slopes.float()[:, None, None] * dist[None]
+        vis = (dist >= 0) & (dist < window)
+        sc = sc.masked_fill(~vis[None], float("-inf"))
+        w = torch.softmax(sc, dim=-1)
+        if talk is not None:
+            w = torch.einsum("hg,gtj->htj", talk.float(), w)
+        ve = vv.repeat_interleave(rep, dim=1)                                   # [ctx, H, dv]
+        o = torch.einsum("htj,jhd->thd", w, ve)
+        out[t0:t1] = o.reshape(t1 - t0, H * dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(out_dtype or q.dtype)
+
+
+def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, positions, H, d, dv,
+          out_dtype):
+    """proj fp32 [T, 2*H*d + H*dv] = [qz | fz | v]; state fp32 [slots, H, d, dv] updated in
+    place; a portion whose first position is 0 starts from zero. See csrc/kernels/recurrent.hip."""
+    T = proj.shape[0]
+    out = torch.zeros(T, H * dv, dtype=torch.float32, device=proj.device)
+    cu = cu_seqlens.tolist()
+    sl = slots.tolist()
+    low = lower.float().reshape(H, d)
+    fb = f_bias.float().reshape(H, d)
+    nw = norm_w.float()
+    for s in range(len(cu) - 1):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0 or sl[s] < 0:
+            continue
+        S = state[sl[s]].clone()
+        if int(positions[t0]) == 0:
+            S.zero_()
+        p = proj[t0:t1].float()
+        qv = F.silu(p[:, :H * d]).reshape(-1, H, d)
+        fv = low + (1.0 - low) * torch.sigmoid(p[:, H * d:2 * H * d].reshape(-1, H, d) + fb)
+        vv = p[:, 2 * H * d:2 * H * d + H * dv].reshape(-1, H, dv)
+        for t in range(t1 - t0):
+            S = fv[t][:, :, None] * S + (1.0 - fv[t])[:, :, None] * vv[t][:, None, :]
+            o = torch.einsum("hdv,hd->hv", S, qv[t])
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * nw
+            out[t0 + t] = o.reshape(H * dv)
+        state[sl[s]] = S
+    return out.to(out_dtype)
