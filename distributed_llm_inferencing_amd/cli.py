@@ -33,6 +33,9 @@ launcher for an 8-GPU MI355X box.
                     node 0 serves the model
     loadgen         --master URL --model M [--requests N] [--concurrency C | --rate R]
                     end-to-end load through the master API: tokens/s, p50/p99 latency
+    trace-run       --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+                    replay a token trace from stdin through the engine's steps and write the
+                    logits at the wanted places (engine/replay.py; also ``bin/trace_run``)
     bench           ... (bench.py)
 """
 from __future__ import annotations
@@ -347,6 +350,9 @@ def main(argv=None):
         return _join_pipeline(rest)
     if cmd == "loadgen":
         from .loadgen import main as m
+        return m(rest)
+    if cmd == "trace-run":
+        from .engine.replay import main as m
         return m(rest)
     if cmd == "bench":
         root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
