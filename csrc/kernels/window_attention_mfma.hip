@@ -1,0 +1,320 @@
+// MFMA form of the windowed attention of window_attention.hip (same arguments, same options,
+// bf16 storage): one workgroup of 8 waves per (sequence, tile of 16 consecutive query tokens,
+// 128-wide slice of the value dimension), all heads in the workgroup because the head-mixing
+// matrix needs every head's normalised weights at the same (query, key).
+//
+// Two passes over the window in tiles of 32 keys:
+//   pass 1   S^T = K . Q^T per head (v_mfma_f32_16x16x32_bf16, K rows as operand A, so a lane
+//            holds 8 keys of ONE query: max / sum reduce over 2 shuffles), running max m and
+//            sum l per (head, query) in registers.
+//   pass 2   S^T again, w = exp(s - m) / l, stored bf16 as Pm[(query, key)][head]; the mix
+//            W' = talk . W is an MFMA with talk as operand A and Pm rows as operand B; W'
+//            lands as Pp[head][query][key]; then O += W' . V with W' rows as operand A and the
+//            V tile, staged transposed (Vt[dim][key]), as operand B.
+// Heads are dealt to waves round-robin (head h -> wave h % 8, at most 4 heads a wave, H <= 32);
+// the key / value tiles are staged per group of kv heads that fits the LDS budget. Query
+// fragments are re-read from global memory (L2) per use: with 576-wide latent queries they do
+// not fit registers, and the LDS is taken by the weight tiles.
+//
+// Masked positions (outside the window, after the query, past the sequence, rows past the
+// tile's last query) get weight 0; a query row always sees itself, so l > 0.
+#include "common.h"
+
+namespace {
+
+constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8;
+
+struct MfmaArgs {
+  const u16* q; int ldq;
+  const u16* k; long k_stride;
+  const u16* v; long v_stride;
+  u16* out; int ldo;
+  const float* gate; int ldg;
+  const float* slopes;
+  const float* talk;
+  const int* cu; const int* positions;
+  const int* block_tables; int bt_stride; int block_size;
+  int H, G, dq, dv, window;
+  float scale;
+  int Hp;        // H rounded up to 32 (mix K dimension)
+  int CG;        // kv heads staged per step
+};
+
+__device__ __forceinline__ float group4_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+__device__ __forceinline__ float group4_sum(float v) {
+  v += __shfl_xor(v, 16, 64);
+  return v + __shfl_xor(v, 32, 64);
+}
+
+__global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int H = a.H, G = a.G, dq = a.dq, dv = a.dv, Hp = a.Hp, CG = a.CG;
+  const int ldk = dq + 8;                         // padded K row (elements)
+  const int dvo = blockIdx.z * 128;               // value slice of this workgroup
+  const int dvc = min(128, dv - dvo);
+  const int dvb = dvc >> 4;
+  u16* Ks = (u16*)smem;                           // [CG][TK][ldk]
+  u16* Vt = Ks + CG * TK * ldk;                   // [CG][128][40]
+  u16* Pm = Vt + CG * 128 * 40;                   // [TQ*TK][Hp]
+  u16* Pp = Pm + TQ * TK * Hp;                    // [H][TQ][40]
+  u16* Tk = Pp + H * TQ * 40;                     // [Hp16][Hp] talk in bf16, zero padded
+  int* slot = (int*)(Tk + ((H + 15) & ~15) * Hp); // [TK]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int fr = lane & 15, fq = lane >> 4;
+  const int s = blockIdx.y;
+  const int t0 = a.cu[s] + blockIdx.x * TQ;
+  const int t_end = a.cu[s + 1];
+  if (t0 >= t_end) return;
+  const int nq = min(TQ, t_end - t0);
+  const int p0 = a.positions[t0];                 // positions of a portion are consecutive
+  const int p_last = p0 + nq - 1;
+  const int lo = max(0, p0 - a.window + 1);
+  const int ntiles = (p_last - lo) / TK + 1;
+  const int* bt = a.block_tables + (long)s * a.bt_stride;
+  const int hpg = H / G;
+  const int my_p = p0 + fr;                       // this lane's query position (column fr)
+  const bool my_q = fr < nq;
+  const bool has_talk = a.talk != nullptr;
+  const int Hp16 = (H + 15) & ~15;
+
+  if (has_talk) {
+    for (int i = tid; i < Hp16 * Hp; i += 512) {
+      const int h = i / Hp, g = i % Hp;
+      Tk[i] = (h < H && g < H) ? f2bf(a.talk[h * H + g]) : (u16)0;
+    }
+  }
+  // zero the mix operand once: head columns [H, Hp) stay zero for the whole kernel
+  if (has_talk)
+    for (int i = tid; i < TQ * TK * Hp / 2; i += 512) ((uint32_t*)Pm)[i] = 0u;
+
+  float m_run[MAXHW], l_run[MAXHW];
+  f32x4 oacc[MAXHW][MAXDVB];
+#pragma unroll
+  for (int hh = 0; hh < MAXHW; ++hh) {
+    m_run[hh] = -INFINITY;
+    l_run[hh] = 0.f;
+#pragma unroll
+    for (int b = 0; b < MAXDVB; ++b) oacc[hh][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int nf = dq >> 5;                         // 32-wide K-steps of the score product
+
+  for (int pass = 0; pass < 2; ++pass) {
+    for (int tile = 0; tile < ntiles; ++tile) {
+      const int j0 = lo + tile * TK;
+      __syncthreads();                            // previous tile's readers are done
+      if (tid < TK) {
+        const int j = j0 + tid;
+        slot[tid] = j <= p_last ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
+      }
+      for (int c0 = 0; c0 < G; c0 += CG) {
+        const int cg = min(CG, G - c0);
+        __syncthreads();                          // slot table ready; Ks free
+        {                                         // stage K tiles of kv heads [c0, c0+cg)
+          const int cpr = dq >> 3;                // 16-byte chunks per row
+          const int total = cg * TK * cpr;
+          for (int i = tid; i < total; i += 512) {
+            const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
+            uint4 val = {0u, 0u, 0u, 0u};
+            const int sl = slot[r];
+            if (sl >= 0)
+              val = *reinterpret_cast<const uint4*>(a.k + (long)sl * a.k_stride +
+                                                    (long)(c0 + c) * dq + ch * 8);
+            *reinterpret_cast<uint4*>(Ks + ((long)c * TK + r) * ldk + ch * 8) = val;
+          }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int hh = 0; hh < MAXHW; ++hh) {
+          const int h = wave + hh * NW;
+          if (h >= H) continue;
+          const int c = h / hpg;
+          if (c < c0 || c >= c0 + cg) continue;
+          const u16* kt = Ks + (long)(c - c0) * TK * ldk;
+          f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+          const u16* qrow = a.q + (long)(t0 + fr) * a.ldq + (long)h * dq + fq * 8;
+          for (int f = 0; f < nf; ++f) {
+            uint4 qv = {0u, 0u, 0u, 0u};
+            if (my_q) qv = *reinterpret_cast<const uint4*>(qrow + f * 32);
+            const bf16x8 qf = *reinterpret_cast<const bf16x8*>(&qv);
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+              const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+                  kt + (long)(kb * 16 + fr) * ldk + f * 32 + fq * 8);
+              sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf, sacc[kb], 0, 0, 0);
+            }
+          }
+          // lane: query fr, keys j0 + kb*16 + 4*fq + r
+          const float slope = a.slopes ? a.slopes[h] : 0.f;
+          float sv[8];
+          float tmax = -INFINITY;
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int j = j0 + kb * 16 + fq * 4 + r;
+              const int dist = my_p - j;
+              float x = sacc[kb][r] * a.scale - slope * (float)dist;
+              if (!my_q || dist < 0 || dist >= a.window) x = -INFINITY;
+              sv[kb * 4 + r] = x;
+              tmax = fmaxf(tmax, x);
+            }
+          if (pass == 0) {
+            tmax = group4_max(tmax);
+            const float m_new = fmaxf(m_run[hh], tmax);
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum += sv[i] == -INFINITY ? 0.f : expf(sv[i] - m_new);
+            sum = group4_sum(sum);
+            const float carry = m_run[hh] == -INFINITY ? 0.f : l_run[hh] * expf(m_run[hh] - m_new);
+            l_run[hh] = carry + sum;
+            m_run[hh] = m_new;
+          } else {
+            const float inv = l_run[hh] > 0.f ? 1.f / l_run[hh] : 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const float x = sv[kb * 4 + r];
+                const float w = x == -INFINITY ? 0.f : expf(x - m_run[hh]) * inv;
+                const int key = kb * 16 + fq * 4 + r;
+                if (has_talk) Pm[(long)(fr * TK + key) * Hp + h] = f2bf(w);
+                else Pp[((long)h * TQ + fr) * 40 + key] = f2bf(w);
+              }
+          }
+        }
+      }
+      if (pass == 0) continue;
+      if (has_talk) {
+        __syncthreads();                          // every head's weights are in Pm
+        // W'[h][x] = sum_g talk[h][g] Pm[x][g]: jobs = (h block, x block of 16)
+        const int nxb = TQ * TK / 16, jobs = (Hp16 >> 4) * nxb;
+        for (int job = wave; job < jobs; job += NW) {
+          const int hb = job / nxb, xb = job % nxb;
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+          for (int kk = 0; kk < Hp; kk += 32) {
+            const bf16x8 tf = *reinterpret_cast<const bf16x8*>(
+                Tk + (long)(hb * 16 + fr) * Hp + kk + fq * 8);
+            const bf16x8 pf = *reinterpret_cast<const bf16x8*>(
+                Pm + (long)(xb * 16 + fr) * Hp + kk + fq * 8);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf, pf, acc, 0, 0, 0);
+          }
+          // lane: heads hb*16 + 4*fq + r, x = xb*16 + fr  (x = query * TK + key)
+          const int x = xb * 16 + fr, qi = x / TK, key = x % TK;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int h = hb * 16 + fq * 4 + r;
+            if (h < H) Pp[((long)h * TQ + qi) * 40 + key] = f2bf(acc[r]);
+          }
+        }
+      }
+      // O += W' . V per group of kv heads
+      for (int c0 = 0; c0 < G; c0 += CG) {
+        const int cg = min(CG, G - c0);
+        __syncthreads();                          // Pp complete (first step) / Vt free
+        {
+          const int cpr = dvc >> 3;
+          const int total = cg * TK * cpr;
+          for (int i = tid; i < total; i += 512) {
+            const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
+            uint4 val = {0u, 0u, 0u, 0u};
+            const int sl = slot[r];
+            if (sl >= 0)
+              val = *reinterpret_cast<const uint4*>(a.v + (long)sl * a.v_stride +
+                                                    (long)(c0 + c) * dv + dvo + ch * 8);
+            const u16* e = reinterpret_cast<const u16*>(&val);
+            u16* dst = Vt + ((long)c * 128 + ch * 8) * 40 + r;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) dst[u * 40] = e[u];
+          }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int hh = 0; hh < MAXHW; ++hh) {
+          const int h = wave + hh * NW;
+          if (h >= H) continue;
+          const int c = h / hpg;
+          if (c < c0 || c >= c0 + cg) continue;
+          const bf16x8 pf = *reinterpret_cast<const bf16x8*>(
+              Pp + ((long)h * TQ + fr) * 40 + fq * 8);
+          const u16* vt = Vt + (long)(c - c0) * 128 * 40;
+#pragma unroll
+          for (int b = 0; b < MAXDVB; ++b) {
+            if (b >= dvb) continue;
+            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (long)(b * 16 + fr) * 40 + fq * 8);
+            // operand A = V^T rows (dim), operand B = W' rows (query): lane holds dims
+            // b*16 + 4*fq + r of query fr
+            oacc[hh][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, oacc[hh][b], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if (!my_q) return;
+#pragma unroll
+  for (int hh = 0; hh < MAXHW; ++hh) {
+    const int h = wave + hh * NW;
+    if (h >= H) continue;
+#pragma unroll
+    for (int b = 0; b < MAXDVB; ++b) {
+      if (b >= dvb) continue;
+      const int col = h * dv + dvo + b * 16 + fq * 4;
+      float o[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        o[r] = oacc[hh][b][r];
+        if (a.gate != nullptr)
+          o[r] *= 1.f / (1.f + expf(-a.gate[(long)(t0 + fr) * a.ldg + col + r]));
+      }
+      uint2 pk;
+      pk.x = pack2bf(o[0], o[1]);
+      pk.y = pack2bf(o[2], o[3]);
+      *reinterpret_cast<uint2*>(a.out + (long)(t0 + fr) * a.ldo + col) = pk;
+    }
+  }
+}
+
+}  // namespace
+
+// Returns hipErrorNotSupported (801) when the shapes do not fit this form; the caller then
+// runs the scalar kernel.
+extern "C" int dli_window_attention_mfma(
+    const void* q, int ldq, const void* k, long k_stride, const void* v, long v_stride, void* out,
+    int ldo, const float* gate, int ldg, const float* slopes, const float* talk, const int* cu,
+    const int* positions, const int* block_tables, int bt_stride, int block_size, int num_seqs,
+    int max_seqlen, int H, int G, int dq, int dv, int window, float scale, hipStream_t st) {
+  if (num_seqs <= 0 || max_seqlen <= 0) return 0;
+  const bool aligned = (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 &&
+                       (uintptr_t)out % 8 == 0 && ldq % 8 == 0 && k_stride % 8 == 0 &&
+                       v_stride % 8 == 0 && ldo % 4 == 0;
+  if (H < 1 || H > NW * MAXHW || G < 1 || H % G || dq % 32 || dv % 16 || !aligned || window < 1 ||
+      block_size < 1)
+    return (int)hipErrorNotSupported;
+  const int Hp = (H + 31) & ~31, Hp16 = (H + 15) & ~15;
+  const int ldk = dq + 8;
+  const size_t fixed = ((size_t)TQ * TK * Hp + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
+                       TK * 4 + 64;
+  const size_t per_cg = ((size_t)TK * ldk + 128 * 40) * 2;
+  const size_t budget = 150 * 1024;
+  if (fixed + per_cg > budget) return (int)hipErrorNotSupported;
+  int CG = (int)((budget - fixed) / per_cg);
+  CG = CG > G ? G : CG;
+  CG = CG > NW ? NW : CG;
+  const size_t sh = fixed + CG * per_cg;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)window_attention_mfma_kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return (int)e;
+    raised = true;
+  }
+  MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
+             ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
+             H, G, dq, dv, window, scale, Hp, CG};
+  dim3 grid((max_seqlen + TQ - 1) / TQ, num_seqs, (dv + 127) / 128);
+  window_attention_mfma_kernel<<<grid, 512, sh, st>>>(a);
+  DLI_RETURN_LAUNCH();
+}

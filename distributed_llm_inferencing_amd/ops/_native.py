@@ -81,6 +81,8 @@ _SIGS = {
     "dli_mla_prepare": [P, I, P, F, I, I, I, I, I, I, P, P, P, P, P, P, I, P],
     "dli_window_attention": [P, I, P, L, P, L, P, I, P, I, P, P, P, P, P,
                              I, I, I, I, I, I, I, I, I, F, I, P],
+    "dli_window_attention_mfma": [P, I, P, L, P, L, P, I, P, I, P, P, P, P, P,
+                                  I, I, I, I, I, I, I, I, I, F, P],
     "dli_hgrn2": [P, I, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, P],
 }
 

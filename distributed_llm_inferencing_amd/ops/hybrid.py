@@ -10,6 +10,7 @@ exact mode) is the dtype of the weights; kernels take it as ``dt``.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -20,6 +21,9 @@ from . import reference as R
 
 _call = N.call
 _p = N.ptr
+_NOT_SUPPORTED = 801            # hipErrorNotSupported: a launcher declining a shape
+# DLI_WINATTN_SCALAR=1 keeps bf16 windowed attention on the scalar kernel (A/B, debugging)
+MFMA_ATTENTION = os.environ.get("DLI_WINATTN_SCALAR", "0") != "1"
 
 
 def _dt(dtype: torch.dtype) -> int:
@@ -191,6 +195,18 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
     T = q.shape[0]
     S = cu_seqlens.shape[0] - 1
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    if q.dtype == torch.bfloat16 and MFMA_ATTENTION:
+        # the MFMA form; shapes it does not take (odd head sizes, > 32 heads) fall through
+        rc = N.require_native().dli_window_attention_mfma(
+            _p(q), q.stride(0), _p(k_cache), k_cache.stride(0), _p(v_cache), v_cache.stride(0),
+            _p(out), out.stride(0), _p(gate), gate.stride(0) if gate is not None else 0,
+            _p(slopes), _p(talk), _p(cu_seqlens), _p(positions), _p(block_tables),
+            block_tables.stride(0), block_size, S, int(max_seqlen), H, G, dq, dv, int(window),
+            float(scale), _st())
+        if rc == 0:
+            return out
+        if rc != _NOT_SUPPORTED:
+            raise RuntimeError(f"dli_window_attention_mfma failed with hipError {rc}")
     _call("dli_window_attention", _p(q), q.stride(0), _p(k_cache), k_cache.stride(0),
           _p(v_cache), v_cache.stride(0), _p(out), out.stride(0), _p(gate),
           gate.stride(0) if gate is not None else 0, _p(slopes), _p(talk), _p(cu_seqlens),

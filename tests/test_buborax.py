@@ -327,3 +327,76 @@ def test_config_reader_reads_every_size():
     c["layers"][0]["type"] = "convolution"
     with pytest.raises(ValueError):
         config_from_hf(c)
+
+
+# ------------------------------------------------------------------ MFMA attention kernel
+def _paged_case(lens, starts, H, G, dq, dv, block, shared_kv, seed, dtype=torch.bfloat16):
+    """Random queries of portions [start, start+len) per sequence over shuffled pages."""
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    ctx = [s + n for s, n in zip(starts, lens)]
+    nblk = [-(-c // block) for c in ctx]
+    total = sum(nblk) + 3
+    perm = torch.randperm(total, generator=g).tolist()
+    tables = torch.zeros(S, max(nblk), dtype=torch.int32)
+    at = 0
+    for s in range(S):
+        tables[s, :nblk[s]] = torch.tensor(perm[at:at + nblk[s]], dtype=torch.int32)
+        at += nblk[s]
+    kw = G * dq
+    k_cache = torch.randn(total * block, kw, generator=g).to(dtype)
+    v_cache = k_cache if shared_kv else torch.randn(total * block, G * dv, generator=g).to(dtype)
+    T = sum(lens)
+    q = torch.randn(T, H * dq, generator=g).to(dtype)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    pos = torch.cat([torch.arange(s, s + n, dtype=torch.int32) for s, n in zip(starts, lens)])
+    return q, k_cache, v_cache, cu, pos, tables
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,dq,dv,win,talk,shared", [
+    (4, 2, 32, 32, 24, True, False), (8, 8, 64, 64, 100, True, False),
+    (32, 8, 128, 128, 70, True, False), (5, 1, 96, 64, 33, False, True),
+    (16, 1, 160, 144, 64, False, True), (3, 3, 32, 32, 1, True, False)])
+def test_mfma_window_attention_matches_reference(gpu, H, G, dq, dv, win, talk, shared):
+    from distributed_llm_inferencing_amd.ops import hybrid as Hy
+    from distributed_llm_inferencing_amd.ops import reference as R
+    lens, starts = [37, 1, 16, 5, 1], [0, 63, 48, 200, 0]
+    block = 16
+    q, kc, vc, cu, pos, bt = _paged_case(lens, starts, H, G, dq, dv, block, shared, seed=H + dq)
+    g = torch.Generator().manual_seed(1)
+    T = q.shape[0]
+    slopes = torch.pow(2.0, -8.0 * torch.arange(1, H + 1) / H).float() if talk else None
+    tk = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)).to(torch.bfloat16).float() if talk else None
+    gate = torch.randn(T, H * dv + 7, generator=g)[:, :H * dv] if talk else None
+    scale = 1.0 / dq ** 0.5
+    want = R.window_attention(q, kc, vc, dq, dv, H, G, cu, pos, bt, block, win, scale, slopes, tk,
+                              gate, out_dtype=torch.float32)
+    d = lambda t: None if t is None else t.to(gpu)      # noqa: E731
+    args = (d(q), d(kc), d(kc) if shared else d(vc), dq, dv, H, G, d(cu), max(lens), d(pos),
+            d(bt), block, win, scale, d(slopes), d(tk), d(gate))
+    assert Hy.MFMA_ATTENTION
+    got = Hy.window_attention(*args).float().cpu()
+    Hy.MFMA_ATTENTION = False
+    try:
+        scalar = Hy.window_attention(*args).float().cpu()
+    finally:
+        Hy.MFMA_ATTENTION = True
+    lim = 0.03 * want.abs().max().item() + 0.02
+    assert (scalar - want).abs().max() < lim
+    assert (got - want).abs().max() < lim
+    assert not torch.equal(got, scalar) or H * dq < 64      # the two kernels really differ
+
+
+@pytest.mark.gpu
+def test_model_on_mfma_sized_heads(gpu):
+    """A whole model whose head sizes take the MFMA attention path, cut in portions."""
+    c = config([attn(heads=4, kv=2, dim=32, win=20, ff=64), hgrn(heads=2, dim=16, vdim=32),
+                latent(heads=4, dim=16, rot_dim=16, vdim=16, rank=48, win=18, dims=8)],
+               width=64, groups=2, loop=(0, 2, 2))
+    w = O.random_weights(c, seed=31)
+    t = toks(60, c["vocab"], 5)
+    want = O.forward(c, w, t)
+    eng = engine(c, w, "cuda", torch.bfloat16)
+    close(replay(eng, t, [60]), want, torch.bfloat16, "whole")
+    close(replay(eng, t, [17, 1, 1, 30, 2, 9]), want, torch.bfloat16, "portions")
