@@ -67,6 +67,88 @@ def _like_for_like_value():
         return None
 
 
+def run_design(a):
+    """``--design buborax``: prefill and decode throughput of the hybrid design at layer sizes
+    of a real model (random weights), beside a Llama of equal width, depth (= layer runs),
+    head sizes and feed-forward width, both through ``LLMEngine.generate``. One JSON line."""
+    from dataclasses import replace
+    from distributed_llm_inferencing_amd.engine import SamplingParams
+    from distributed_llm_inferencing_amd.engine.llm_engine import LLMEngine
+    from distributed_llm_inferencing_amd.models.configs import LayerSpec, get_config, hybrid_config
+    D, Fw, V, Hh, G, hd = a.design_width, a.design_ff, 32000, a.design_width // 128, 8, 128
+    win = a.design_window
+    specs = (LayerSpec("attention", heads=Hh, kv_heads=G, dim=hd, vdim=hd, window=win,
+                       scale=hd ** -0.5, ff=Fw),
+             LayerSpec("hgrn2", heads=Hh, dim=hd, vdim=hd, ff=Fw),
+             LayerSpec("latent_attention", heads=Hh, kv_heads=1, dim=hd, vdim=hd, window=win,
+                       scale=(hd + 64) ** -0.5, rot_dim=64, kv_rank=512, rot_dims=64, ff=Fw),
+             LayerSpec("attention", heads=Hh, kv_heads=G, dim=hd, vdim=hd, window=win,
+                       scale=hd ** -0.5, ff=Fw))
+    hyb = hybrid_config("buborax-bench", D, V, specs, loop=(1, 3, 2), norm_groups=4,
+                        residual_mult=0.7)
+    runs = len(hyb.layer_runs())
+    llama = replace(get_config("llama3-8b"), name="llama-bench", hidden_size=D, num_layers=runs,
+                    num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw,
+                    vocab_size=V, max_position=1 << 16)
+    rng = np.random.default_rng(0)
+    out = {}
+    for cfg in (hyb, llama):
+        res = {}
+        for (S, L) in a.design_prefill:
+            eng = LLMEngine(cfg, device="cuda:0", max_batch=max(S, 8), max_model_len=L + 64,
+                            block_size=16, max_kv_tokens=S * (L + 64) + 4096,
+                            max_prefill_tokens=S * L, use_graphs=False, lookahead=False)
+            prompts = [rng.integers(0, V, L).tolist() for _ in range(S)]
+            sp = SamplingParams(max_new_tokens=1, ignore_eos=True)
+            ts = []
+            for _ in range(a.warmup + a.steps):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                eng.generate(prompts, sp)
+                torch.cuda.synchronize()
+                ts.append(time.perf_counter() - t0)
+            t = min(ts[a.warmup:])
+            res[f"prefill_{S}x{L}_tok_s"] = round(S * L / t, 1)
+            del eng
+            torch.cuda.empty_cache()
+        for (B, C) in a.design_decode:
+            n_new = 33
+            eng = LLMEngine(cfg, device="cuda:0", max_batch=B, max_model_len=C + n_new + 16,
+                            block_size=16, max_kv_tokens=B * (C + n_new + 32) + 4096,
+                            max_prefill_tokens=max(8192, C))
+            eng.warmup(buckets=[B])
+            prompts = [rng.integers(0, V, C).tolist() for _ in range(B)]
+
+            def wave(n):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                eng.generate(prompts, SamplingParams(max_new_tokens=n, ignore_eos=True))
+                torch.cuda.synchronize()
+                return time.perf_counter() - t0
+            wave(2)
+            best = None
+            for _ in range(max(1, a.steps)):
+                t1, tn = wave(1), wave(n_new)
+                d = (tn - t1) / (n_new - 1)
+                best = d if best is None else min(best, d)
+            res[f"decode_b{B}_ctx{C}_tok_s"] = round(B / best, 1)
+            res[f"decode_b{B}_ctx{C}_ms_per_step"] = round(1000 * best, 3)
+            del eng
+            torch.cuda.empty_cache()
+        out[cfg.name] = res
+    print(json.dumps({"metric": "prefill and decode tokens/s, Buborax design vs Llama of equal "
+                                "size (random weights)", "unit": "tokens/s", "n_gpus": 1,
+                      "dtype": "bf16", "data": "synthetic prompts, random-init weights",
+                      "config": {"width": D, "ff": Fw, "layer_runs": runs, "heads": Hh,
+                                 "kv_heads": G, "head_dim": hd, "window": win,
+                                 "latent_rank": 512},
+                      "results": out}), flush=True)
+
+
+def _pairs(text):
+    return [tuple(int(v) for v in p.split("x")) for p in text.split(",") if p]
+
+
 def _heartbeat(period_s: float = 45.0):
     """A stderr line every ``period_s`` on rank 0 (stdout keeps the one JSON line): engine
     start-up (weights, autotune, graph capture) and an 8-stage run can stay silent for
@@ -198,7 +280,20 @@ def main():
                     help="N>1: pp = layer-sharded pipeline (dense, default), ep = expert "
                          "parallel (MoE), tp = tensor-parallel ablation, dp = independent "
                          "replicas")
+    ap.add_argument("--design", default=None, choices=["buborax"],
+                    help="instead of the headline workload: prefill / decode throughput of "
+                         "this design at real layer sizes beside a Llama of equal size")
+    ap.add_argument("--design-width", type=int, default=4096)
+    ap.add_argument("--design-ff", type=int, default=14336)
+    ap.add_argument("--design-window", type=int, default=1024)
+    ap.add_argument("--design-prefill", type=_pairs, default=_pairs("4x2048,32x256"),
+                    help="prompts x tokens, comma separated")
+    ap.add_argument("--design-decode", type=_pairs, default=_pairs("64x1024,8x2048"),
+                    help="batch x context, comma separated")
     a = ap.parse_args()
+    if a.design:
+        _heartbeat()
+        return run_design(a)
 
     from distributed_llm_inferencing_amd import launch
     if a.gpus > 1 and not launch.under_launcher():
