@@ -93,6 +93,8 @@ def run_design(a):
     rng = np.random.default_rng(0)
     out = {}
     for cfg in (hyb, llama):
+        if cfg.name.split("-")[0] not in a.design_models.split(","):
+            continue
         res = {}
         for (S, L) in a.design_prefill:
             eng = LLMEngine(cfg, device="cuda:0", max_batch=max(S, 8), max_model_len=L + 64,
@@ -283,6 +285,7 @@ def main():
     ap.add_argument("--design", default=None, choices=["buborax"],
                     help="instead of the headline workload: prefill / decode throughput of "
                          "this design at real layer sizes beside a Llama of equal size")
+    ap.add_argument("--design-models", default="buborax,llama", help="which of the two to run")
     ap.add_argument("--design-width", type=int, default=4096)
     ap.add_argument("--design-ff", type=int, default=14336)
     ap.add_argument("--design-window", type=int, default=1024)

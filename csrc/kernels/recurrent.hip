@@ -11,9 +11,10 @@
 // reused without clearing). Sequences with slot < 0 (padding rows of a captured decode step)
 // are skipped.
 //
-// This is the sequential form: one workgroup per (head, sequence), thread c owns column c of
-// the state, which lives in LDS for the whole portion. It is what a decode step needs (one
-// token: the state is read and written once); long portions pay one pass per token.
+// Two kernels, one workgroup per (head, sequence), thread c owns column c of the state: decode
+// steps stream the state through registers (read once, written once); portions keep it in
+// LDS and walk their tokens in chunks (the walk is sequential in time by the recurrence's
+// per-channel decay; the gates and the norm of a chunk are computed in parallel).
 #include "common.h"
 
 namespace {
@@ -25,6 +26,12 @@ template <typename S> __device__ __forceinline__ void stf(S* p, float v);
 template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 
+constexpr int TC = 16;   // tokens per chunk of the portion kernel
+
+// Portions: the state of one (sequence, head) lives in LDS for the whole portion; tokens are
+// taken in chunks of TC: (1) every thread helps turning the chunk's q / f pre-activations into
+// silu(q) and the forget gate, (2) thread c walks the chunk's tokens over its state column
+// without any barrier, (3) the chunk's read-outs are RMS-normed, one wave per token.
 template <typename S>
 __global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* __restrict__ f_bias,
                              const S* __restrict__ lower, const S* __restrict__ norm_w, float eps,
@@ -33,9 +40,9 @@ __global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* _
                              S* __restrict__ out, int ldo, int H, int d, int dv) {
   extern __shared__ float sm[];
   float* St = sm;                 // [d][dv]
-  float* qv = St + d * dv;        // [d] silu(qz)
-  float* fv = qv + d;             // [d] forget gate
-  float* red = fv + d;            // [16]
+  float* qv = St + d * dv;        // [TC][d] silu(qz)
+  float* fv = qv + TC * d;        // [TC][d] forget gate
+  float* ov = fv + TC * d;        // [TC][dv] read-outs of the chunk
   const int h = blockIdx.x, s = blockIdx.y;
   const int slot = slots[s];
   const int t0 = cu[s], t1 = cu[s + 1];
@@ -49,34 +56,109 @@ __global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* _
   float* sp = state + ((long)slot * H + h) * d * dv;
   const bool fresh = positions[t0] == 0;
   for (int i = c; i < d * dv; i += blockDim.x) St[i] = fresh ? 0.f : sp[i];
-  const float nw = c < dv ? ldf(norm_w + c) : 0.f;
-  for (int t = t0; t < t1; ++t) {
-    const float* row = proj + (long)t * ldp;
-    __syncthreads();
-    for (int i = c; i < d; i += blockDim.x) {
-      const float qz = row[h * d + i];
+  const int lane = c & 63, wid = c >> 6, nw = blockDim.x >> 6;
+  for (int tc = t0; tc < t1; tc += TC) {
+    const int n = min(TC, t1 - tc);
+    __syncthreads();                     // previous chunk's norm phase is done with ov
+    for (int i = c; i < n * d; i += blockDim.x) {
+      const int tt = i / d, k = i % d;
+      const float* row = proj + (long)(tc + tt) * ldp;
+      const float qz = row[h * d + k];
       qv[i] = qz / (1.f + expf(-qz));
-      const float lw = ldf(lower + h * d + i);
-      const float fz = row[H * d + h * d + i] + ldf(f_bias + h * d + i);
+      const float lw = ldf(lower + h * d + k);
+      const float fz = row[H * d + h * d + k] + ldf(f_bias + h * d + k);
       fv[i] = lw + (1.f - lw) / (1.f + expf(-fz));
     }
     __syncthreads();
-    float o = 0.f;
     if (c < dv) {
-      const float v = row[2 * H * d + h * dv + c];
-      for (int i = 0; i < d; ++i) {
-        const float f = fv[i];
-        const float sv = f * St[i * dv + c] + (1.f - f) * v;
-        St[i * dv + c] = sv;
-        o += sv * qv[i];
+      for (int tt = 0; tt < n; ++tt) {
+        const float v = proj[(long)(tc + tt) * ldp + 2 * H * d + h * dv + c];
+        const float* q = qv + tt * d;
+        const float* f = fv + tt * d;
+        float o = 0.f;
+        for (int i = 0; i < d; ++i) {
+          const float fi = f[i];
+          const float sv = fi * St[i * dv + c] + (1.f - fi) * v;
+          St[i * dv + c] = sv;
+          o += sv * q[i];
+        }
+        ov[tt * dv + c] = o;
       }
     }
-    const float ss = block_sum(o * o, red);
-    if (c < dv)
-      stf(out + (long)t * ldo + h * dv + c, o * (1.f / sqrtf(ss / (float)dv + eps)) * nw);
+    __syncthreads();
+    for (int tt = wid; tt < n; tt += nw) {
+      float ss = 0.f;
+      for (int k = lane; k < dv; k += 64) { const float o = ov[tt * dv + k]; ss += o * o; }
+      ss = wave_sum(ss);
+      const float rs = 1.f / sqrtf(ss / (float)dv + eps);
+      for (int k = lane; k < dv; k += 64)
+        stf(out + (long)(tc + tt) * ldo + h * dv + k, ov[tt * dv + k] * rs * ldf(norm_w + k));
+    }
   }
   __syncthreads();
   for (int i = c; i < d * dv; i += blockDim.x) sp[i] = St[i];
+}
+
+// Decode steps (every sequence brings one token): the state streams through registers, one
+// read and one write per element, no LDS copy. One workgroup per (head, sequence), thread c
+// owns column c: consecutive threads touch consecutive addresses of every state row.
+template <typename S>
+__global__ void hgrn2_step_kernel(const float* __restrict__ proj, int ldp,
+                                  const S* __restrict__ f_bias, const S* __restrict__ lower,
+                                  const S* __restrict__ norm_w, float eps,
+                                  float* __restrict__ state, const int* __restrict__ slots,
+                                  const int* __restrict__ cu, const int* __restrict__ positions,
+                                  S* __restrict__ out, int ldo, int H, int d, int dv) {
+  extern __shared__ float sm[];
+  float* qv = sm;                 // [d]
+  float* fv = qv + d;             // [d]
+  float* red = fv + d;            // [16]
+  const int h = blockIdx.x, s = blockIdx.y;
+  const int slot = slots[s];
+  const int t = cu[s];
+  const int c = threadIdx.x;
+  if (cu[s + 1] <= t) return;
+  if (slot < 0) {
+    if (c < dv) stf(out + (long)t * ldo + h * dv + c, 0.f);
+    return;
+  }
+  const float* row = proj + (long)t * ldp;
+  for (int k = c; k < d; k += blockDim.x) {
+    const float qz = row[h * d + k];
+    qv[k] = qz / (1.f + expf(-qz));
+    const float lw = ldf(lower + h * d + k);
+    const float fz = row[H * d + h * d + k] + ldf(f_bias + h * d + k);
+    fv[k] = lw + (1.f - lw) / (1.f + expf(-fz));
+  }
+  __syncthreads();
+  const bool fresh = positions[t] == 0;
+  float o = 0.f;
+  if (c < dv) {
+    float* sp = state + ((long)slot * H + h) * d * dv + c;
+    const float v = row[2 * H * d + h * dv + c];
+    int i = 0;
+    for (; i + 8 <= d; i += 8) {          // 8 independent loads in flight per thread
+      float old[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) old[u] = fresh ? 0.f : sp[(long)(i + u) * dv];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float fi = fv[i + u];
+        const float sv = fi * old[u] + (1.f - fi) * v;
+        sp[(long)(i + u) * dv] = sv;
+        o += sv * qv[i + u];
+      }
+    }
+    for (; i < d; ++i) {
+      const float fi = fv[i];
+      const float sv = fi * (fresh ? 0.f : sp[(long)i * dv]) + (1.f - fi) * v;
+      sp[(long)i * dv] = sv;
+      o += sv * qv[i];
+    }
+  }
+  const float ss = block_sum(o * o, red);
+  if (c < dv)
+    stf(out + (long)t * ldo + h * dv + c, o * (1.f / sqrtf(ss / (float)dv + eps)) * ldf(norm_w + c));
 }
 
 }  // namespace
@@ -84,10 +166,26 @@ __global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* _
 extern "C" int dli_hgrn2(const float* proj, int ldp, const void* f_bias, const void* lower,
                          const void* norm_w, float eps, float* state, const int* slots,
                          const int* cu, const int* positions, void* out, int ldo, int num_seqs,
-                         int H, int d, int dv, int dt, hipStream_t st) {
+                         int max_seqlen, int H, int d, int dv, int dt, hipStream_t st) {
   if (num_seqs <= 0) return 0;
   const int threads = ((dv + 63) / 64) * 64;
-  const size_t sh = ((size_t)d * dv + 2 * d + 16) * 4;
+  if (H < 1 || d < 1 || dv < 1 || threads > 1024) return (int)hipErrorInvalidValue;
+  if (max_seqlen == 1) {                 // a decode step: stream the state, no LDS copy
+    dim3 grid1(H, num_seqs);
+    const size_t sh1 = ((size_t)2 * d + 16) * 4;
+    if (sh1 > 48 * 1024) return (int)hipErrorInvalidValue;
+    if (dt == 0)
+      hgrn2_step_kernel<u16><<<grid1, threads, sh1, st>>>(
+          proj, ldp, (const u16*)f_bias, (const u16*)lower, (const u16*)norm_w, eps, state, slots,
+          cu, positions, (u16*)out, ldo, H, d, dv);
+    else if (dt == 1)
+      hgrn2_step_kernel<float><<<grid1, threads, sh1, st>>>(
+          proj, ldp, (const float*)f_bias, (const float*)lower, (const float*)norm_w, eps, state,
+          slots, cu, positions, (float*)out, ldo, H, d, dv);
+    else return (int)hipErrorInvalidValue;
+    DLI_RETURN_LAUNCH();
+  }
+  const size_t sh = ((size_t)d * dv + 2 * TC * d + TC * dv) * 4;
   if (H < 1 || d < 1 || dv < 1 || threads > 1024 || sh > 160 * 1024)
     return (int)hipErrorInvalidValue;
   if (sh > 48 * 1024) {

@@ -38,6 +38,13 @@ struct MfmaArgs {
   float scale;
   int Hp;        // H rounded up to 32 (mix K dimension)
   int CG;        // kv heads staged per step
+  // key-split form (few query tiles, long windows: decode steps): the window's tiles are dealt
+  // to nsplit workgroups; mode 1 = pass 1 only (partial max / sum -> stats_ws), mode 2 = pass 2
+  // only (the partials combined first; un-gated fp32 partial outputs -> o_ws), mode 0 = both
+  int mode, nsplit, ndvs;
+  float* stats_ws;   // [S][q tiles][nsplit][H][TQ][2]
+  float* o_ws;       // [nsplit][T][H*dv]
+  long o_ws_stride;  // T * H * dv
 };
 
 __device__ __forceinline__ float group4_max(float v) {
@@ -53,7 +60,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int H = a.H, G = a.G, dq = a.dq, dv = a.dv, Hp = a.Hp, CG = a.CG;
   const int ldk = dq + 8;                         // padded K row (elements)
-  const int dvo = blockIdx.z * 128;               // value slice of this workgroup
+  const int dvo = (blockIdx.z % a.ndvs) * 128;    // value slice of this workgroup
+  const int split = blockIdx.z / a.ndvs;
   const int dvc = min(128, dv - dvo);
   const int dvb = dvc >> 4;
   u16* Ks = (u16*)smem;                           // [CG][TK][ldk]
@@ -101,9 +109,34 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
     for (int b = 0; b < MAXDVB; ++b) oacc[hh][b] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int nf = dq >> 5;                         // 32-wide K-steps of the score product
+  int tile_lo = 0, tile_hi = ntiles;
+  if (a.nsplit > 1) {
+    const int per = (ntiles + a.nsplit - 1) / a.nsplit;
+    tile_lo = split * per;
+    tile_hi = min(ntiles, tile_lo + per);
+  }
+  const long stats_base = ((long)s * gridDim.x + blockIdx.x) * a.nsplit;
+  if (a.mode == 2) {                              // global max / sum from every split's pair
+#pragma unroll
+    for (int hh = 0; hh < MAXHW; ++hh) {
+      const int h = wave + hh * NW;
+      if (h >= H) continue;
+      float M = -INFINITY;
+      for (int k2 = 0; k2 < a.nsplit; ++k2)
+        M = fmaxf(M, a.stats_ws[(((stats_base + k2) * H + h) * TQ + fr) * 2]);
+      float L = 0.f;
+      for (int k2 = 0; k2 < a.nsplit; ++k2) {
+        const float* pr = a.stats_ws + (((stats_base + k2) * H + h) * TQ + fr) * 2;
+        if (pr[0] != -INFINITY) L += pr[1] * expf(pr[0] - M);
+      }
+      m_run[hh] = M;
+      l_run[hh] = L;
+    }
+  }
+  const int pass_lo = a.mode == 2 ? 1 : 0, pass_hi = a.mode == 1 ? 1 : 2;
 
-  for (int pass = 0; pass < 2; ++pass) {
-    for (int tile = 0; tile < ntiles; ++tile) {
+  for (int pass = pass_lo; pass < pass_hi; ++pass) {
+    for (int tile = tile_lo; tile < tile_hi; ++tile) {
       const int j0 = lo + tile * TK;
       __syncthreads();                            // previous tile's readers are done
       if (tid < TK) {
@@ -253,7 +286,35 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
       }
     }
   }
+  if (a.mode == 1) {
+    if (fq == 0) {
+#pragma unroll
+      for (int hh = 0; hh < MAXHW; ++hh) {
+        const int h = wave + hh * NW;
+        if (h >= H) continue;
+        float* pr = a.stats_ws + (((stats_base + split) * H + h) * TQ + fr) * 2;
+        pr[0] = m_run[hh];
+        pr[1] = l_run[hh];
+      }
+    }
+    return;
+  }
   if (!my_q) return;
+  if (a.mode == 2) {
+#pragma unroll
+    for (int hh = 0; hh < MAXHW; ++hh) {
+      const int h = wave + hh * NW;
+      if (h >= H) continue;
+#pragma unroll
+      for (int b = 0; b < MAXDVB; ++b) {
+        if (b >= dvb) continue;
+        const int col = h * dv + dvo + b * 16 + fq * 4;
+        *reinterpret_cast<f32x4*>(a.o_ws + (long)split * a.o_ws_stride +
+                                  (long)(t0 + fr) * H * dv + col) = oacc[hh][b];
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int hh = 0; hh < MAXHW; ++hh) {
     const int h = wave + hh * NW;
@@ -277,7 +338,49 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   }
 }
 
+// out[t][c] = bf16(gate * sum over splits of the partial outputs), 4 columns a thread
+__global__ void __launch_bounds__(256) split_reduce_kernel(
+    u16* __restrict__ out, int ldo, const float* __restrict__ o_ws, long stride, int nsplit,
+    const float* __restrict__ gate, int ldg, int T, int width) {
+  const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int w4 = width >> 2;
+  if (gid >= (long)T * w4) return;
+  const int t = (int)(gid / w4), c = (int)(gid % w4) * 4;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < nsplit; ++k)
+    acc += *reinterpret_cast<const f32x4*>(o_ws + k * stride + (long)t * width + c);
+  if (gate != nullptr) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] *= 1.f / (1.f + expf(-gate[(long)t * ldg + c + r]));
+  }
+  uint2 pk;
+  pk.x = pack2bf(acc[0], acc[1]);
+  pk.y = pack2bf(acc[2], acc[3]);
+  *reinterpret_cast<uint2*>(out + (long)t * ldo + c) = pk;
+}
+
 }  // namespace
+
+// Workspace bytes the key-split form may use for a step of T rows in num_seqs sequences
+// (0: the step will not be split).
+static int pick_splits(int num_seqs, int max_seqlen, int dv, int window) {
+  const int qtiles = (max_seqlen + TQ - 1) / TQ, ndvs = (dv + 127) / 128;
+  const long base = (long)qtiles * num_seqs * ndvs;
+  const int ntiles_max = (window + TQ - 2) / TK + 2;
+  if (base >= 256 || ntiles_max < 4) return 1;
+  long n = 512 / base;
+  if (n > 16) n = 16;
+  if (n > ntiles_max / 2) n = ntiles_max / 2;
+  return n < 2 ? 1 : (int)n;
+}
+
+extern "C" long dli_window_attention_mfma_workspace_bytes(int num_seqs, int max_seqlen, int T,
+                                                          int H, int dv, int window) {
+  const int nsplit = pick_splits(num_seqs, max_seqlen, dv, window);
+  if (nsplit == 1) return 0;
+  const long qtiles = (max_seqlen + TQ - 1) / TQ;
+  return ((long)num_seqs * qtiles * nsplit * H * TQ * 2 + (long)nsplit * T * H * dv) * 4;
+}
 
 // Returns hipErrorNotSupported (801) when the shapes do not fit this form; the caller then
 // runs the scalar kernel.
@@ -285,7 +388,8 @@ extern "C" int dli_window_attention_mfma(
     const void* q, int ldq, const void* k, long k_stride, const void* v, long v_stride, void* out,
     int ldo, const float* gate, int ldg, const float* slopes, const float* talk, const int* cu,
     const int* positions, const int* block_tables, int bt_stride, int block_size, int num_seqs,
-    int max_seqlen, int H, int G, int dq, int dv, int window, float scale, hipStream_t st) {
+    int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int T, void* ws,
+    hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
   const bool aligned = (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 &&
                        (uintptr_t)out % 8 == 0 && ldq % 8 == 0 && k_stride % 8 == 0 &&
@@ -311,10 +415,29 @@ extern "C" int dli_window_attention_mfma(
     if (e != hipSuccess) return (int)e;
     raised = true;
   }
+  const int ndvs = (dv + 127) / 128, qtiles = (max_seqlen + TQ - 1) / TQ;
+  const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, dv, window) : 1;
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
-             H, G, dq, dv, window, scale, Hp, CG};
-  dim3 grid((max_seqlen + TQ - 1) / TQ, num_seqs, (dv + 127) / 128);
-  window_attention_mfma_kernel<<<grid, 512, sh, st>>>(a);
+             H, G, dq, dv, window, scale, Hp, CG, 0, 1, ndvs, nullptr, nullptr, 0};
+  if (nsplit == 1) {
+    dim3 grid(qtiles, num_seqs, ndvs);
+    window_attention_mfma_kernel<<<grid, 512, sh, st>>>(a);
+    DLI_RETURN_LAUNCH();
+  }
+  if (T <= 0 || (H * dv) % 4 || ldo % 4) return (int)hipErrorInvalidValue;
+  a.nsplit = nsplit;
+  a.stats_ws = (float*)ws;
+  a.o_ws = a.stats_ws + (long)num_seqs * qtiles * nsplit * H * TQ * 2;
+  a.o_ws_stride = (long)T * H * dv;
+  a.mode = 1;
+  a.ndvs = 1;                                     // the statistics do not depend on the slice
+  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, nsplit), 512, sh, st>>>(a);
+  a.mode = 2;
+  a.ndvs = ndvs;
+  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, ndvs * nsplit), 512, sh, st>>>(a);
+  const long quads = (long)T * (H * dv / 4);
+  split_reduce_kernel<<<(int)((quads + 255) / 256), 256, 0, st>>>(
+      (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv);
   DLI_RETURN_LAUNCH();
 }

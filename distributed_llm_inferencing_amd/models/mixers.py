@@ -67,7 +67,8 @@ def hgrn2_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float)
     (state,) = cache
     proj = H.linear_any(h, lp["w_in"])                       # fp32 [T, q | f | v]
     o = H.hgrn2(proj, lp["f_b"], lp["lower"], lp["o_norm"], eps, state, step.state_slots,
-                step.cu_seqlens, step.positions, spec.heads, spec.dim, spec.vdim)
+                step.cu_seqlens, step.max_seqlen, step.positions, spec.heads, spec.dim,
+                spec.vdim)
     return H.linear_any(o, lp["wo"])
 
 

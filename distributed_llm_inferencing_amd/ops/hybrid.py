@@ -197,12 +197,16 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
     if q.dtype == torch.bfloat16 and MFMA_ATTENTION:
         # the MFMA form; shapes it does not take (odd head sizes, > 32 heads) fall through
-        rc = N.require_native().dli_window_attention_mfma(
+        lib = N.require_native()
+        nb = lib.dli_window_attention_mfma_workspace_bytes(S, int(max_seqlen), T, H, dv,
+                                                           int(window))
+        ws = G.workspace(q.device, nb) if nb else None       # key-split form (decode steps)
+        rc = lib.dli_window_attention_mfma(
             _p(q), q.stride(0), _p(k_cache), k_cache.stride(0), _p(v_cache), v_cache.stride(0),
             _p(out), out.stride(0), _p(gate), gate.stride(0) if gate is not None else 0,
             _p(slopes), _p(talk), _p(cu_seqlens), _p(positions), _p(block_tables),
             block_tables.stride(0), block_size, S, int(max_seqlen), H, G, dq, dv, int(window),
-            float(scale), _st())
+            float(scale), T, _p(ws), _st())
         if rc == 0:
             return out
         if rc != _NOT_SUPPORTED:
@@ -215,7 +219,8 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
     return out
 
 
-def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, positions, H, d, dv):
+def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, max_seqlen, positions,
+          H, d, dv):
     dtype = norm_w.dtype
     if not proj.is_cuda:
         return R.hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, positions,
@@ -224,6 +229,6 @@ def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, positions,
     S = cu_seqlens.shape[0] - 1
     out = torch.empty(T, H * dv, dtype=dtype, device=proj.device)
     _call("dli_hgrn2", _p(proj), proj.stride(0), _p(f_bias), _p(lower), _p(norm_w), float(eps),
-          _p(state), _p(slots), _p(cu_seqlens), _p(positions), _p(out), out.stride(0), S, H, d,
-          dv, _dt(dtype), _st())
+          _p(state), _p(slots), _p(cu_seqlens), _p(positions), _p(out), out.stride(0), S,
+          int(max_seqlen), H, d, dv, _dt(dtype), _st())
     return out
