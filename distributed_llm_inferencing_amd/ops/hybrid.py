@@ -16,7 +16,7 @@ from typing import Optional
 import torch
 
 from . import _native as N
-from . import gemm as G
+from . import gemm as _gemm
 from . import reference as R
 
 _call = N.call
@@ -200,7 +200,7 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
         lib = N.require_native()
         nb = lib.dli_window_attention_mfma_workspace_bytes(S, int(max_seqlen), T, H, dv,
                                                            int(window))
-        ws = G.workspace(q.device, nb) if nb else None       # key-split form (decode steps)
+        ws = _gemm.workspace(q.device, nb) if nb else None       # key-split form (decode steps)
         rc = lib.dli_window_attention_mfma(
             _p(q), q.stride(0), _p(k_cache), k_cache.stride(0), _p(v_cache), v_cache.stride(0),
             _p(out), out.stride(0), _p(gate), gate.stride(0) if gate is not None else 0,
