@@ -121,18 +121,27 @@ def run_design(a):
             eng.warmup(buckets=[B])
             prompts = [rng.integers(0, V, C).tolist() for _ in range(B)]
 
-            def wave(n):
+            def decode_steps(n):
+                """Admit the batch, run its prefill, then time n pure decode steps."""
+                sp = SamplingParams(max_new_tokens=n + 8, ignore_eos=True)
+                for p in prompts:
+                    eng.add_request(p, sp)
+                sch = eng.scheduler
+                while sch.waiting or any(sch.prefilling):
+                    eng.step()
+                for _ in range(3):
+                    eng.step()
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
-                eng.generate(prompts, SamplingParams(max_new_tokens=n, ignore_eos=True))
+                for _ in range(n):
+                    eng.step()
                 torch.cuda.synchronize()
-                return time.perf_counter() - t0
-            wave(2)
-            best = None
-            for _ in range(max(1, a.steps)):
-                t1, tn = wave(1), wave(n_new)
-                d = (tn - t1) / (n_new - 1)
-                best = d if best is None else min(best, d)
+                dt = (time.perf_counter() - t0) / n
+                while eng.has_work():
+                    eng.step()
+                return dt
+            decode_steps(4)
+            best = min(decode_steps(n_new - 1) for _ in range(max(1, a.steps)))
             res[f"decode_b{B}_ctx{C}_tok_s"] = round(B / best, 1)
             res[f"decode_b{B}_ctx{C}_ms_per_step"] = round(1000 * best, 3)
             del eng

@@ -32,15 +32,17 @@ constexpr int TC = 16;   // tokens per chunk of the portion kernel
 // taken in chunks of TC: (1) every thread helps turning the chunk's q / f pre-activations into
 // silu(q) and the forget gate, (2) thread c walks the chunk's tokens over its state column
 // without any barrier, (3) the chunk's read-outs are RMS-normed, one wave per token.
-template <typename S>
-__global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* __restrict__ f_bias,
+// D > 0: the state column of thread c lives in D registers (d == D, fully unrolled walk);
+// D == 0: any d, the state lives in LDS.
+template <typename S, int D>
+__global__ void __launch_bounds__(D ? 256 : 1024) hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* __restrict__ f_bias,
                              const S* __restrict__ lower, const S* __restrict__ norm_w, float eps,
                              float* __restrict__ state, const int* __restrict__ slots,
                              const int* __restrict__ cu, const int* __restrict__ positions,
                              S* __restrict__ out, int ldo, int H, int d, int dv) {
-  extern __shared__ float sm[];
-  float* St = sm;                 // [d][dv]
-  float* qv = St + d * dv;        // [TC][d] silu(qz)
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  float* St = sm;                 // [d][dv] (D == 0 only)
+  float* qv = St + (D ? 0 : d * dv);   // [TC][d] silu(qz)
   float* fv = qv + TC * d;        // [TC][d] forget gate
   float* ov = fv + TC * d;        // [TC][dv] read-outs of the chunk
   const int h = blockIdx.x, s = blockIdx.y;
@@ -55,7 +57,13 @@ __global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* _
   if (t1 <= t0) return;
   float* sp = state + ((long)slot * H + h) * d * dv;
   const bool fresh = positions[t0] == 0;
-  for (int i = c; i < d * dv; i += blockDim.x) St[i] = fresh ? 0.f : sp[i];
+  float reg[D ? D : 1];
+  if (D) {
+#pragma unroll
+    for (int i = 0; i < D; ++i) reg[i] = (fresh || c >= dv) ? 0.f : sp[(long)i * dv + c];
+  } else {
+    for (int i = c; i < d * dv; i += blockDim.x) St[i] = fresh ? 0.f : sp[i];
+  }
   const int lane = c & 63, wid = c >> 6, nw = blockDim.x >> 6;
   for (int tc = t0; tc < t1; tc += TC) {
     const int n = min(TC, t1 - tc);
@@ -76,11 +84,24 @@ __global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* _
         const float* q = qv + tt * d;
         const float* f = fv + tt * d;
         float o = 0.f;
-        for (int i = 0; i < d; ++i) {
-          const float fi = f[i];
-          const float sv = fi * St[i * dv + c] + (1.f - fi) * v;
-          St[i * dv + c] = sv;
-          o += sv * q[i];
+        if (D) {
+#pragma unroll
+          for (int i = 0; i < D; i += 4) {
+            const f32x4 f4 = *reinterpret_cast<const f32x4*>(f + i);
+            const f32x4 q4 = *reinterpret_cast<const f32x4*>(q + i);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              reg[i + u] = f4[u] * reg[i + u] + (1.f - f4[u]) * v;
+              o += reg[i + u] * q4[u];
+            }
+          }
+        } else {
+          for (int i = 0; i < d; ++i) {
+            const float fi = f[i];
+            const float sv = fi * St[i * dv + c] + (1.f - fi) * v;
+            St[i * dv + c] = sv;
+            o += sv * q[i];
+          }
         }
         ov[tt * dv + c] = o;
       }
@@ -94,6 +115,13 @@ __global__ void hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* _
       for (int k = lane; k < dv; k += 64)
         stf(out + (long)(tc + tt) * ldo + h * dv + k, ov[tt * dv + k] * rs * ldf(norm_w + k));
     }
+  }
+  if (D) {
+    if (c < dv) {
+#pragma unroll
+      for (int i = 0; i < D; ++i) sp[(long)i * dv + c] = reg[i];
+    }
+    return;
   }
   __syncthreads();
   for (int i = c; i < d * dv; i += blockDim.x) sp[i] = St[i];
@@ -185,29 +213,33 @@ extern "C" int dli_hgrn2(const float* proj, int ldp, const void* f_bias, const v
     else return (int)hipErrorInvalidValue;
     DLI_RETURN_LAUNCH();
   }
-  const size_t sh = ((size_t)d * dv + 2 * TC * d + TC * dv) * 4;
-  if (H < 1 || d < 1 || dv < 1 || threads > 1024 || sh > 160 * 1024)
-    return (int)hipErrorInvalidValue;
-  if (sh > 48 * 1024) {
-    static bool raised[2] = {false, false};
-    if (dt >= 0 && dt < 2 && !raised[dt]) {
-      const void* fn = dt == 0 ? (const void*)hgrn2_kernel<u16> : (const void*)hgrn2_kernel<float>;
-      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         160 * 1024);
-      if (e != hipSuccess) return (int)e;
-      raised[dt] = true;
-    }
-  }
+  const int D = ((d == 16 || d == 32 || d == 64 || d == 128) && threads <= 256) ? d : 0;
+  const size_t sh = ((size_t)(D ? 0 : d * dv) + 2 * TC * d + TC * dv) * 4;
+  if (sh > 160 * 1024) return (int)hipErrorInvalidValue;
   dim3 grid(H, num_seqs);
-  if (dt == 0)
-    hgrn2_kernel<u16><<<grid, threads, sh, st>>>(proj, ldp, (const u16*)f_bias, (const u16*)lower,
-                                                 (const u16*)norm_w, eps, state, slots, cu,
-                                                 positions, (u16*)out, ldo, H, d, dv);
-  else if (dt == 1)
-    hgrn2_kernel<float><<<grid, threads, sh, st>>>(proj, ldp, (const float*)f_bias,
-                                                   (const float*)lower, (const float*)norm_w, eps,
-                                                   state, slots, cu, positions, (float*)out, ldo,
-                                                   H, d, dv);
+#define HGRN2_LAUNCH(ST, DD)                                                                   \
+  do {                                                                                         \
+    if (sh > 48 * 1024) {                                                                      \
+      hipError_t e = hipFuncSetAttribute((const void*)hgrn2_kernel<ST, DD>,                    \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
+      if (e != hipSuccess) return (int)e;                                                      \
+    }                                                                                          \
+    hgrn2_kernel<ST, DD><<<grid, threads, sh, st>>>(                                           \
+        proj, ldp, (const ST*)f_bias, (const ST*)lower, (const ST*)norm_w, eps, state, slots,  \
+        cu, positions, (ST*)out, ldo, H, d, dv);                                               \
+  } while (0)
+#define HGRN2_BY_D(ST)                                \
+  do {                                                \
+    switch (D) {                                      \
+      case 16: HGRN2_LAUNCH(ST, 16); break;           \
+      case 32: HGRN2_LAUNCH(ST, 32); break;           \
+      case 64: HGRN2_LAUNCH(ST, 64); break;           \
+      case 128: HGRN2_LAUNCH(ST, 128); break;         \
+      default: HGRN2_LAUNCH(ST, 0); break;            \
+    }                                                 \
+  } while (0)
+  if (dt == 0) HGRN2_BY_D(u16);
+  else if (dt == 1) HGRN2_BY_D(float);
   else return (int)hipErrorInvalidValue;
   DLI_RETURN_LAUNCH();
 }

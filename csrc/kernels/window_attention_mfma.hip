@@ -22,7 +22,7 @@
 
 namespace {
 
-constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8;
+constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8, STG = 4;
 
 struct MfmaArgs {
   const u16* q; int ldq;
@@ -149,14 +149,28 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         {                                         // stage K tiles of kv heads [c0, c0+cg)
           const int cpr = dq >> 3;                // 16-byte chunks per row
           const int total = cg * TK * cpr;
-          for (int i = tid; i < total; i += 512) {
-            const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
-            uint4 val = {0u, 0u, 0u, 0u};
-            const int sl = slot[r];
-            if (sl >= 0)
-              val = *reinterpret_cast<const uint4*>(a.k + (long)sl * a.k_stride +
-                                                    (long)(c0 + c) * dq + ch * 8);
-            *reinterpret_cast<uint4*>(Ks + ((long)c * TK + r) * ldk + ch * 8) = val;
+          for (int base = 0; base < total; base += 512 * STG) {
+            uint4 val[STG];                       // STG loads in flight per thread
+#pragma unroll
+            for (int u = 0; u < STG; ++u) {
+              const int i = base + u * 512 + tid;
+              val[u] = uint4{0u, 0u, 0u, 0u};
+              if (i < total) {
+                const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
+                const int sl = slot[r];
+                if (sl >= 0)
+                  val[u] = *reinterpret_cast<const uint4*>(a.k + (long)sl * a.k_stride +
+                                                           (long)(c0 + c) * dq + ch * 8);
+              }
+            }
+#pragma unroll
+            for (int u = 0; u < STG; ++u) {
+              const int i = base + u * 512 + tid;
+              if (i < total) {
+                const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
+                *reinterpret_cast<uint4*>(Ks + ((long)c * TK + r) * ldk + ch * 8) = val[u];
+              }
+            }
           }
         }
         __syncthreads();
@@ -169,15 +183,23 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
           const u16* kt = Ks + (long)(c - c0) * TK * ldk;
           f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
           const u16* qrow = a.q + (long)(t0 + fr) * a.ldq + (long)h * dq + fq * 8;
-          for (int f = 0; f < nf; ++f) {
-            uint4 qv = {0u, 0u, 0u, 0u};
-            if (my_q) qv = *reinterpret_cast<const uint4*>(qrow + f * 32);
-            const bf16x8 qf = *reinterpret_cast<const bf16x8*>(&qv);
+          for (int f0 = 0; f0 < nf; f0 += 4) {     // 4 query fragments in flight
+            uint4 qv[4];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-              const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
-                  kt + (long)(kb * 16 + fr) * ldk + f * 32 + fq * 8);
-              sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf, sacc[kb], 0, 0, 0);
+            for (int u = 0; u < 4; ++u) {
+              qv[u] = uint4{0u, 0u, 0u, 0u};
+              if (my_q && f0 + u < nf) qv[u] = *reinterpret_cast<const uint4*>(qrow + (f0 + u) * 32);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              if (f0 + u >= nf) continue;
+              const bf16x8 qf = *reinterpret_cast<const bf16x8*>(&qv[u]);
+#pragma unroll
+              for (int kb = 0; kb < 2; ++kb) {
+                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+                    kt + (long)(kb * 16 + fr) * ldk + (f0 + u) * 32 + fq * 8);
+                sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf, sacc[kb], 0, 0, 0);
+              }
             }
           }
           // lane: query fr, keys j0 + kb*16 + 4*fq + r
@@ -251,17 +273,33 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         {
           const int cpr = dvc >> 3;
           const int total = cg * TK * cpr;
-          for (int i = tid; i < total; i += 512) {
-            const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
-            uint4 val = {0u, 0u, 0u, 0u};
-            const int sl = slot[r];
-            if (sl >= 0)
-              val = *reinterpret_cast<const uint4*>(a.v + (long)sl * a.v_stride +
-                                                    (long)(c0 + c) * dv + dvo + ch * 8);
-            const u16* e = reinterpret_cast<const u16*>(&val);
-            u16* dst = Vt + ((long)c * 128 + ch * 8) * 40 + r;
+          for (int base = 0; base < total; base += 512 * STG) {
+            uint4 val[STG];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) dst[u * 40] = e[u];
+            for (int u = 0; u < STG; ++u) {
+              const int i = base + u * 512 + tid;
+              val[u] = uint4{0u, 0u, 0u, 0u};
+              if (i < total) {
+                // consecutive threads take consecutive keys of one 8-dim chunk: their
+                // transposed 2-byte stores then fall into consecutive LDS addresses
+                const int r = i % TK, ch = (i / TK) % cpr, c = i / (TK * cpr);
+                const int sl = slot[r];
+                if (sl >= 0)
+                  val[u] = *reinterpret_cast<const uint4*>(a.v + (long)sl * a.v_stride +
+                                                           (long)(c0 + c) * dv + dvo + ch * 8);
+              }
+            }
+#pragma unroll
+            for (int u = 0; u < STG; ++u) {
+              const int i = base + u * 512 + tid;
+              if (i < total) {
+                const int r = i % TK, ch = (i / TK) % cpr, c = i / (TK * cpr);
+                const u16* e = reinterpret_cast<const u16*>(&val[u]);
+                u16* dst = Vt + ((long)c * 128 + ch * 8) * 40 + r;
+#pragma unroll
+                for (int w = 0; w < 8; ++w) dst[w * 40] = e[w];
+              }
+            }
           }
         }
         __syncthreads();

@@ -98,10 +98,13 @@ def toks(n, vocab, seed=1):
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("layer", [attn(ff=0), attn(heads=6, kv=1, dim=8, win=3, ff=0),
                                    hgrn(ff=0), hgrn(heads=1, dim=24, vdim=5, ff=0),
+                                   hgrn(heads=2, dim=64, vdim=20, ff=0),
+                                   hgrn(heads=1, dim=128, vdim=72, ff=0),
                                    latent(), latent(heads=1, dim=4, rot_dim=6, vdim=3, rank=5,
                                                     win=4, dims=6),
                                    attn(heads=2, kv=2, dim=8, win=50, ff=40)],
-                         ids=["attn", "attn_mqa", "hgrn2", "hgrn2_1head", "latent", "latent_odd",
+                         ids=["attn", "attn_mqa", "hgrn2", "hgrn2_1head", "hgrn2_d64", "hgrn2_d128",
+                              "latent", "latent_odd",
                               "ff"])
 def test_mechanism_alone(layer, device, dtype):
     c = config([layer], groups=1, mult=1.0)
