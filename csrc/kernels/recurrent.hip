@@ -68,19 +68,39 @@ __global__ void __launch_bounds__(D ? 256 : 1024) hgrn2_kernel(const float* __re
   for (int tc = t0; tc < t1; tc += TC) {
     const int n = min(TC, t1 - tc);
     __syncthreads();                     // previous chunk's norm phase is done with ov
-    for (int i = c; i < n * d; i += blockDim.x) {
-      const int tt = i / d, k = i % d;
-      const float* row = proj + (long)(tc + tt) * ldp;
-      const float qz = row[h * d + k];
-      qv[i] = qz / (1.f + expf(-qz));
-      const float lw = ldf(lower + h * d + k);
-      const float fz = row[H * d + h * d + k] + ldf(f_bias + h * d + k);
-      fv[i] = lw + (1.f - lw) / (1.f + expf(-fz));
+    for (int i0 = c; i0 < n * d; i0 += 4 * blockDim.x) {
+      float qz[4], fz[4];                // 8 loads in flight per thread
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * blockDim.x;
+        qz[u] = fz[u] = 0.f;
+        if (i < n * d) {
+          const float* row = proj + (long)(tc + i / d) * ldp + h * d + i % d;
+          qz[u] = row[0];
+          fz[u] = row[H * d];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * blockDim.x;
+        if (i < n * d) {
+          const int k = i % d;
+          qv[i] = qz[u] / (1.f + expf(-qz[u]));
+          const float lw = ldf(lower + h * d + k);
+          fv[i] = lw + (1.f - lw) / (1.f + expf(-(fz[u] + ldf(f_bias + h * d + k))));
+        }
+      }
     }
     __syncthreads();
     if (c < dv) {
-      for (int tt = 0; tt < n; ++tt) {
-        const float v = proj[(long)(tc + tt) * ldp + 2 * H * d + h * dv + c];
+      float vch[TC];                     // the chunk's values of this column, loads in flight
+#pragma unroll
+      for (int tt = 0; tt < TC; ++tt)
+        vch[tt] = tt < n ? proj[(long)(tc + tt) * ldp + 2 * H * d + h * dv + c] : 0.f;
+#pragma unroll
+      for (int tt = 0; tt < TC; ++tt) {
+        if (tt >= n) break;
+        const float v = vch[tt];
         const float* q = qv + tt * d;
         const float* f = fv + tt * d;
         float o = 0.f;

@@ -11,7 +11,8 @@
 //            W' = talk . W is an MFMA with talk as operand A and Pm rows as operand B; W'
 //            lands as Pp[head][query][key]; then O += W' . V with W' rows as operand A and the
 //            V tile, staged transposed (Vt[dim][key]), as operand B.
-// Heads are dealt to waves round-robin (head h -> wave h % 8, at most 4 heads a wave, H <= 32);
+// With mixing, heads are dealt to waves round-robin (head h -> wave h % 8, at most 4 heads a
+// wave, H <= 32, 128-wide value slices); without it, the wide form takes 8 heads a workgroup;
 // the key / value tiles are staged per group of kv heads that fits the LDS budget. Query
 // fragments are re-read from global memory (L2) per use: with 576-wide latent queries they do
 // not fit registers, and the LDS is taken by the weight tiles.
@@ -42,6 +43,10 @@ struct MfmaArgs {
   // to nsplit workgroups; mode 1 = pass 1 only (partial max / sum -> stats_ws), mode 2 = pass 2
   // only (the partials combined first; un-gated fp32 partial outputs -> o_ws), mode 0 = both
   int mode, nsplit, ndvs;
+  // wide form (no head mixing, so heads need not share a workgroup): 8 heads a workgroup,
+  // one per wave, and the wave's 32 accumulator blocks cover a 512-wide value slice instead
+  // of 4 heads x 128 — latent attention's 512-wide values without recomputing the scores
+  int wide, nhs;
   float* stats_ws;   // [S][q tiles][nsplit][H][TQ][2]
   float* o_ws;       // [nsplit][T][H*dv]
   long o_ws_stride;  // T * H * dv
@@ -60,16 +65,19 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int H = a.H, G = a.G, dq = a.dq, dv = a.dv, Hp = a.Hp, CG = a.CG;
   const int ldk = dq + 8;                         // padded K row (elements)
-  const int dvo = (blockIdx.z % a.ndvs) * 128;    // value slice of this workgroup
-  const int split = blockIdx.z / a.ndvs;
-  const int dvc = min(128, dv - dvo);
+  const bool wide = a.wide != 0;
+  const int dvw = wide ? 512 : 128;               // value slice of a workgroup
+  const int dvo = (blockIdx.z % a.ndvs) * dvw;
+  const int hbase = ((blockIdx.z / a.ndvs) % a.nhs) * NW;
+  const int split = blockIdx.z / (a.ndvs * a.nhs);
+  const int dvc = min(dvw, dv - dvo);
   const int dvb = dvc >> 4;
   u16* Ks = (u16*)smem;                           // [CG][TK][ldk]
-  u16* Vt = Ks + CG * TK * ldk;                   // [CG][128][40]
-  u16* Pm = Vt + CG * 128 * 40;                   // [TQ*TK][Hp]
-  u16* Pp = Pm + TQ * TK * Hp;                    // [H][TQ][40]
-  u16* Tk = Pp + H * TQ * 40;                     // [Hp16][Hp] talk in bf16, zero padded
-  int* slot = (int*)(Tk + ((H + 15) & ~15) * Hp); // [TK]
+  u16* Vt = Ks + CG * TK * ldk;                   // [CG][dvw][40]
+  u16* Pm = Vt + CG * dvw * 40;                   // [TQ*TK][Hp]
+  u16* Pp = Pm + (wide ? 0 : TQ * TK * Hp);       // [H][TQ][40] (wide: [NW][TQ][40], by wave)
+  u16* Tk = Pp + (wide ? NW : H) * TQ * 40;       // [Hp16][Hp] talk in bf16, zero padded
+  int* slot = (int*)(Tk + (wide ? 0 : ((H + 15) & ~15) * Hp));   // [TK]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
@@ -119,8 +127,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   if (a.mode == 2) {                              // global max / sum from every split's pair
 #pragma unroll
     for (int hh = 0; hh < MAXHW; ++hh) {
-      const int h = wave + hh * NW;
-      if (h >= H) continue;
+      const int h = wide ? hbase + wave : wave + hh * NW;
+      if (h >= H || (wide && hh)) continue;
       float M = -INFINITY;
       for (int k2 = 0; k2 < a.nsplit; ++k2)
         M = fmaxf(M, a.stats_ws[(((stats_base + k2) * H + h) * TQ + fr) * 2]);
@@ -176,8 +184,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         __syncthreads();
 #pragma unroll
         for (int hh = 0; hh < MAXHW; ++hh) {
-          const int h = wave + hh * NW;
-          if (h >= H) continue;
+          const int h = wide ? hbase + wave : wave + hh * NW;
+          if (h >= H || (wide && hh)) continue;
           const int c = h / hpg;
           if (c < c0 || c >= c0 + cg) continue;
           const u16* kt = Ks + (long)(c - c0) * TK * ldk;
@@ -237,7 +245,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
                 const float w = x == -INFINITY ? 0.f : expf(x - m_run[hh]) * inv;
                 const int key = kb * 16 + fq * 4 + r;
                 if (has_talk) Pm[(long)(fr * TK + key) * Hp + h] = f2bf(w);
-                else Pp[((long)h * TQ + fr) * 40 + key] = f2bf(w);
+                else Pp[((long)(wide ? wave : h) * TQ + fr) * 40 + key] = f2bf(w);
               }
           }
         }
@@ -295,7 +303,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
               if (i < total) {
                 const int r = i % TK, ch = (i / TK) % cpr, c = i / (TK * cpr);
                 const u16* e = reinterpret_cast<const u16*>(&val[u]);
-                u16* dst = Vt + ((long)c * 128 + ch * 8) * 40 + r;
+                u16* dst = Vt + ((long)c * dvw + ch * 8) * 40 + r;
 #pragma unroll
                 for (int w = 0; w < 8; ++w) dst[w * 40] = e[w];
               }
@@ -305,19 +313,20 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         __syncthreads();
 #pragma unroll
         for (int hh = 0; hh < MAXHW; ++hh) {
-          const int h = wave + hh * NW;
+          const int h = wide ? hbase + wave : wave + hh * NW;
           if (h >= H) continue;
           const int c = h / hpg;
           if (c < c0 || c >= c0 + cg) continue;
           const bf16x8 pf = *reinterpret_cast<const bf16x8*>(
-              Pp + ((long)h * TQ + fr) * 40 + fq * 8);
-          const u16* vt = Vt + (long)(c - c0) * 128 * 40;
+              Pp + ((long)(wide ? wave : h) * TQ + fr) * 40 + fq * 8);
+          const u16* vt = Vt + (long)(c - c0) * dvw * 40;
 #pragma unroll
           for (int b = 0; b < MAXDVB; ++b) {
-            if (b >= dvb) continue;
-            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (long)(b * 16 + fr) * 40 + fq * 8);
+            const int blk = wide ? hh * MAXDVB + b : b;
+            if (blk >= dvb) continue;
+            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (long)(blk * 16 + fr) * 40 + fq * 8);
             // operand A = V^T rows (dim), operand B = W' rows (query): lane holds dims
-            // b*16 + 4*fq + r of query fr
+            // blk*16 + 4*fq + r of query fr
             oacc[hh][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, oacc[hh][b], 0, 0, 0);
           }
         }
@@ -328,8 +337,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
     if (fq == 0) {
 #pragma unroll
       for (int hh = 0; hh < MAXHW; ++hh) {
-        const int h = wave + hh * NW;
-        if (h >= H) continue;
+        const int h = wide ? hbase + wave : wave + hh * NW;
+        if (h >= H || (wide && hh)) continue;
         float* pr = a.stats_ws + (((stats_base + split) * H + h) * TQ + fr) * 2;
         pr[0] = m_run[hh];
         pr[1] = l_run[hh];
@@ -341,12 +350,13 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   if (a.mode == 2) {
 #pragma unroll
     for (int hh = 0; hh < MAXHW; ++hh) {
-      const int h = wave + hh * NW;
+      const int h = wide ? hbase + wave : wave + hh * NW;
       if (h >= H) continue;
 #pragma unroll
       for (int b = 0; b < MAXDVB; ++b) {
-        if (b >= dvb) continue;
-        const int col = h * dv + dvo + b * 16 + fq * 4;
+        const int blk = wide ? hh * MAXDVB + b : b;
+        if (blk >= dvb) continue;
+        const int col = h * dv + dvo + blk * 16 + fq * 4;
         *reinterpret_cast<f32x4*>(a.o_ws + (long)split * a.o_ws_stride +
                                   (long)(t0 + fr) * H * dv + col) = oacc[hh][b];
       }
@@ -355,12 +365,13 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   }
 #pragma unroll
   for (int hh = 0; hh < MAXHW; ++hh) {
-    const int h = wave + hh * NW;
+    const int h = wide ? hbase + wave : wave + hh * NW;
     if (h >= H) continue;
 #pragma unroll
     for (int b = 0; b < MAXDVB; ++b) {
-      if (b >= dvb) continue;
-      const int col = h * dv + dvo + b * 16 + fq * 4;
+      const int blk = wide ? hh * MAXDVB + b : b;
+      if (blk >= dvb) continue;
+      const int col = h * dv + dvo + blk * 16 + fq * 4;
       float o[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -401,9 +412,10 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(
 
 // Workspace bytes the key-split form may use for a step of T rows in num_seqs sequences
 // (0: the step will not be split).
-static int pick_splits(int num_seqs, int max_seqlen, int dv, int window) {
-  const int qtiles = (max_seqlen + TQ - 1) / TQ, ndvs = (dv + 127) / 128;
-  const long base = (long)qtiles * num_seqs * ndvs;
+static int pick_splits(int num_seqs, int max_seqlen, int H, int dv, int window, bool wide) {
+  const int qtiles = (max_seqlen + TQ - 1) / TQ;
+  const int ndvs = wide ? (dv + 511) / 512 : (dv + 127) / 128, nhs = wide ? (H + NW - 1) / NW : 1;
+  const long base = (long)qtiles * num_seqs * ndvs * nhs;
   const int ntiles_max = (window + TQ - 2) / TK + 2;
   if (base >= 256 || ntiles_max < 4) return 1;
   long n = 512 / base;
@@ -413,8 +425,9 @@ static int pick_splits(int num_seqs, int max_seqlen, int dv, int window) {
 }
 
 extern "C" long dli_window_attention_mfma_workspace_bytes(int num_seqs, int max_seqlen, int T,
-                                                          int H, int dv, int window) {
-  const int nsplit = pick_splits(num_seqs, max_seqlen, dv, window);
+                                                          int H, int dv, int window,
+                                                          int mixing) {
+  const int nsplit = pick_splits(num_seqs, max_seqlen, H, dv, window, mixing == 0);
   if (nsplit == 1) return 0;
   const long qtiles = (max_seqlen + TQ - 1) / TQ;
   return ((long)num_seqs * qtiles * nsplit * H * TQ * 2 + (long)nsplit * T * H * dv) * 4;
@@ -432,14 +445,17 @@ extern "C" int dli_window_attention_mfma(
   const bool aligned = (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 &&
                        (uintptr_t)out % 8 == 0 && ldq % 8 == 0 && k_stride % 8 == 0 &&
                        v_stride % 8 == 0 && ldo % 4 == 0;
-  if (H < 1 || H > NW * MAXHW || G < 1 || H % G || dq % 32 || dv % 16 || !aligned || window < 1 ||
-      block_size < 1)
+  const bool wide = talk == nullptr;
+  if (H < 1 || (!wide && H > NW * MAXHW) || G < 1 || H % G || dq % 32 || dv % 16 || !aligned ||
+      window < 1 || block_size < 1)
     return (int)hipErrorNotSupported;
+  const int dvw = wide ? 512 : 128;
   const int Hp = (H + 31) & ~31, Hp16 = (H + 15) & ~15;
   const int ldk = dq + 8;
-  const size_t fixed = ((size_t)TQ * TK * Hp + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
+  const size_t fixed = (wide ? (size_t)NW * TQ * 40
+                             : (size_t)TQ * TK * Hp + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
                        TK * 4 + 64;
-  const size_t per_cg = ((size_t)TK * ldk + 128 * 40) * 2;
+  const size_t per_cg = ((size_t)TK * ldk + (size_t)dvw * 40) * 2;
   const size_t budget = 150 * 1024;
   if (fixed + per_cg > budget) return (int)hipErrorNotSupported;
   int CG = (int)((budget - fixed) / per_cg);
@@ -453,13 +469,15 @@ extern "C" int dli_window_attention_mfma(
     if (e != hipSuccess) return (int)e;
     raised = true;
   }
-  const int ndvs = (dv + 127) / 128, qtiles = (max_seqlen + TQ - 1) / TQ;
-  const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, dv, window) : 1;
+  const int ndvs = (dv + dvw - 1) / dvw, qtiles = (max_seqlen + TQ - 1) / TQ;
+  const int nhs = wide ? (H + NW - 1) / NW : 1;
+  const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, H, dv, window, wide) : 1;
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
-             H, G, dq, dv, window, scale, Hp, CG, 0, 1, ndvs, nullptr, nullptr, 0};
+             H, G, dq, dv, window, scale, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs,
+             nullptr, nullptr, 0};
   if (nsplit == 1) {
-    dim3 grid(qtiles, num_seqs, ndvs);
+    dim3 grid(qtiles, num_seqs, ndvs * nhs);
     window_attention_mfma_kernel<<<grid, 512, sh, st>>>(a);
     DLI_RETURN_LAUNCH();
   }
@@ -470,10 +488,10 @@ extern "C" int dli_window_attention_mfma(
   a.o_ws_stride = (long)T * H * dv;
   a.mode = 1;
   a.ndvs = 1;                                     // the statistics do not depend on the slice
-  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, nsplit), 512, sh, st>>>(a);
+  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, nhs * nsplit), 512, sh, st>>>(a);
   a.mode = 2;
   a.ndvs = ndvs;
-  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, ndvs * nsplit), 512, sh, st>>>(a);
+  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, ndvs * nhs * nsplit), 512, sh, st>>>(a);
   const long quads = (long)T * (H * dv / 4);
   split_reduce_kernel<<<(int)((quads + 255) / 256), 256, 0, st>>>(
       (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv);

@@ -199,7 +199,7 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
         # the MFMA form; shapes it does not take (odd head sizes, > 32 heads) fall through
         lib = N.require_native()
         nb = lib.dli_window_attention_mfma_workspace_bytes(S, int(max_seqlen), T, H, dv,
-                                                           int(window))
+                                                           int(window), int(talk is not None))
         ws = _gemm.workspace(q.device, nb) if nb else None       # key-split form (decode steps)
         rc = lib.dli_window_attention_mfma(
             _p(q), q.stride(0), _p(k_cache), k_cache.stride(0), _p(v_cache), v_cache.stride(0),
