@@ -32,10 +32,12 @@ constexpr int TC = 16;   // tokens per chunk of the portion kernel
 // taken in chunks of TC: (1) every thread helps turning the chunk's q / f pre-activations into
 // silu(q) and the forget gate, (2) thread c walks the chunk's tokens over its state column
 // without any barrier, (3) the chunk's read-outs are RMS-normed, one wave per token.
-// D > 0: the state column of thread c lives in D registers (d == D, fully unrolled walk);
-// D == 0: any d, the state lives in LDS.
-template <typename S, int D>
-__global__ void __launch_bounds__(D ? 256 : 1024) hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* __restrict__ f_bias,
+// D > 0: d == D and the state lives in registers: the block is P groups of dvp = round64(dv)
+// threads, thread (c, part) owns rows [part * D/P, (part+1) * D/P) of column c (fully unrolled
+// walk); the P partial read-outs of a token meet in LDS at the chunk's end.
+// D == 0: any d, the state lives in LDS (P = 1).
+template <typename S, int D, int P>
+__global__ void __launch_bounds__(1024) hgrn2_kernel(const float* __restrict__ proj, int ldp, const S* __restrict__ f_bias,
                              const S* __restrict__ lower, const S* __restrict__ norm_w, float eps,
                              float* __restrict__ state, const int* __restrict__ slots,
                              const int* __restrict__ cu, const int* __restrict__ positions,
@@ -44,31 +46,37 @@ __global__ void __launch_bounds__(D ? 256 : 1024) hgrn2_kernel(const float* __re
   float* St = sm;                 // [d][dv] (D == 0 only)
   float* qv = St + (D ? 0 : d * dv);   // [TC][d] silu(qz)
   float* fv = qv + TC * d;        // [TC][d] forget gate
-  float* ov = fv + TC * d;        // [TC][dv] read-outs of the chunk
+  float* ov = fv + TC * d;        // [P][TC][dv] (partial) read-outs of the chunk
+  float* vv = ov + P * TC * dv;   // [TC][dv] the chunk's values
+  constexpr int R = D ? D / P : 1;
   const int h = blockIdx.x, s = blockIdx.y;
   const int slot = slots[s];
   const int t0 = cu[s], t1 = cu[s + 1];
-  const int c = threadIdx.x;
+  const int dvp = blockDim.x / P;
+  const int c = threadIdx.x % dvp, part = threadIdx.x / dvp;
   if (slot < 0) {                        // padding rows: defined (zero) output, no state
     for (int t = t0; t < t1; ++t)
-      if (c < dv) stf(out + (long)t * ldo + h * dv + c, 0.f);
+      if (c < dv && part == 0) stf(out + (long)t * ldo + h * dv + c, 0.f);
     return;
   }
   if (t1 <= t0) return;
   float* sp = state + ((long)slot * H + h) * d * dv;
   const bool fresh = positions[t0] == 0;
-  float reg[D ? D : 1];
+  float reg[R];
   if (D) {
 #pragma unroll
-    for (int i = 0; i < D; ++i) reg[i] = (fresh || c >= dv) ? 0.f : sp[(long)i * dv + c];
+    for (int i = 0; i < R; ++i)
+      reg[i] = (fresh || c >= dv) ? 0.f : sp[(long)(part * R + i) * dv + c];
   } else {
-    for (int i = c; i < d * dv; i += blockDim.x) St[i] = fresh ? 0.f : sp[i];
+    for (int i = threadIdx.x; i < d * dv; i += blockDim.x) St[i] = fresh ? 0.f : sp[i];
   }
-  const int lane = c & 63, wid = c >> 6, nw = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int tc = t0; tc < t1; tc += TC) {
     const int n = min(TC, t1 - tc);
     __syncthreads();                     // previous chunk's norm phase is done with ov
-    for (int i0 = c; i0 < n * d; i0 += 4 * blockDim.x) {
+    for (int i = threadIdx.x; i < n * dv; i += blockDim.x)
+      vv[i] = proj[(long)(tc + i / dv) * ldp + 2 * H * d + h * dv + i % dv];
+    for (int i0 = threadIdx.x; i0 < n * d; i0 += 4 * blockDim.x) {
       float qz[4], fz[4];                // 8 loads in flight per thread
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -93,22 +101,17 @@ __global__ void __launch_bounds__(D ? 256 : 1024) hgrn2_kernel(const float* __re
     }
     __syncthreads();
     if (c < dv) {
-      float vch[TC];                     // the chunk's values of this column, loads in flight
-#pragma unroll
-      for (int tt = 0; tt < TC; ++tt)
-        vch[tt] = tt < n ? proj[(long)(tc + tt) * ldp + 2 * H * d + h * dv + c] : 0.f;
-#pragma unroll
-      for (int tt = 0; tt < TC; ++tt) {
-        if (tt >= n) break;
-        const float v = vch[tt];
+#pragma unroll 1
+      for (int tt = 0; tt < n; ++tt) {
+        const float v = vv[tt * dv + c];
         const float* q = qv + tt * d;
         const float* f = fv + tt * d;
         float o = 0.f;
         if (D) {
 #pragma unroll
-          for (int i = 0; i < D; i += 4) {
-            const f32x4 f4 = *reinterpret_cast<const f32x4*>(f + i);
-            const f32x4 q4 = *reinterpret_cast<const f32x4*>(q + i);
+          for (int i = 0; i < R; i += 4) {
+            const f32x4 f4 = *reinterpret_cast<const f32x4*>(f + part * R + i);
+            const f32x4 q4 = *reinterpret_cast<const f32x4*>(q + part * R + i);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
               reg[i + u] = f4[u] * reg[i + u] + (1.f - f4[u]) * v;
@@ -123,13 +126,19 @@ __global__ void __launch_bounds__(D ? 256 : 1024) hgrn2_kernel(const float* __re
             o += sv * q[i];
           }
         }
-        ov[tt * dv + c] = o;
+        ov[(part * TC + tt) * dv + c] = o;
       }
     }
     __syncthreads();
     for (int tt = wid; tt < n; tt += nw) {
       float ss = 0.f;
-      for (int k = lane; k < dv; k += 64) { const float o = ov[tt * dv + k]; ss += o * o; }
+      for (int k = lane; k < dv; k += 64) {
+        float o = ov[tt * dv + k];
+#pragma unroll
+        for (int pp = 1; pp < P; ++pp) o += ov[(pp * TC + tt) * dv + k];
+        ov[tt * dv + k] = o;
+        ss += o * o;
+      }
       ss = wave_sum(ss);
       const float rs = 1.f / sqrtf(ss / (float)dv + eps);
       for (int k = lane; k < dv; k += 64)
@@ -139,12 +148,12 @@ __global__ void __launch_bounds__(D ? 256 : 1024) hgrn2_kernel(const float* __re
   if (D) {
     if (c < dv) {
 #pragma unroll
-      for (int i = 0; i < D; ++i) sp[(long)i * dv + c] = reg[i];
+      for (int i = 0; i < R; ++i) sp[(long)(part * R + i) * dv + c] = reg[i];
     }
     return;
   }
   __syncthreads();
-  for (int i = c; i < d * dv; i += blockDim.x) sp[i] = St[i];
+  for (int i = threadIdx.x; i < d * dv; i += blockDim.x) sp[i] = St[i];
 }
 
 // Decode steps (every sequence brings one token): the state streams through registers, one
@@ -233,30 +242,34 @@ extern "C" int dli_hgrn2(const float* proj, int ldp, const void* f_bias, const v
     else return (int)hipErrorInvalidValue;
     DLI_RETURN_LAUNCH();
   }
-  const int D = ((d == 16 || d == 32 || d == 64 || d == 128) && threads <= 256) ? d : 0;
-  const size_t sh = ((size_t)(D ? 0 : d * dv) + 2 * TC * d + TC * dv) * 4;
+  // register form: d in {16, 32, 64, 128}, the state rows dealt to P thread groups
+  int D = (d == 16 || d == 32 || d == 64 || d == 128) ? d : 0;
+  const int P = D >= 64 ? 4 : (D == 32 ? 2 : 1);
+  if (D && threads * P > 1024) D = 0;
+  const int nthreads = D ? threads * P : threads;
+  const size_t sh = ((size_t)(D ? 0 : d * dv) + 2 * TC * d + (size_t)((D ? P : 1) + 1) * TC * dv) * 4;
   if (sh > 160 * 1024) return (int)hipErrorInvalidValue;
   dim3 grid(H, num_seqs);
-#define HGRN2_LAUNCH(ST, DD)                                                                   \
+#define HGRN2_LAUNCH(ST, DD, PP)                                                               \
   do {                                                                                         \
     if (sh > 48 * 1024) {                                                                      \
-      hipError_t e = hipFuncSetAttribute((const void*)hgrn2_kernel<ST, DD>,                    \
+      hipError_t e = hipFuncSetAttribute((const void*)hgrn2_kernel<ST, DD, PP>,                \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
       if (e != hipSuccess) return (int)e;                                                      \
     }                                                                                          \
-    hgrn2_kernel<ST, DD><<<grid, threads, sh, st>>>(                                           \
+    hgrn2_kernel<ST, DD, PP><<<grid, nthreads, sh, st>>>(                                      \
         proj, ldp, (const ST*)f_bias, (const ST*)lower, (const ST*)norm_w, eps, state, slots,  \
         cu, positions, (ST*)out, ldo, H, d, dv);                                               \
   } while (0)
-#define HGRN2_BY_D(ST)                                \
-  do {                                                \
-    switch (D) {                                      \
-      case 16: HGRN2_LAUNCH(ST, 16); break;           \
-      case 32: HGRN2_LAUNCH(ST, 32); break;           \
-      case 64: HGRN2_LAUNCH(ST, 64); break;           \
-      case 128: HGRN2_LAUNCH(ST, 128); break;         \
-      default: HGRN2_LAUNCH(ST, 0); break;            \
-    }                                                 \
+#define HGRN2_BY_D(ST)                                   \
+  do {                                                   \
+    switch (D) {                                         \
+      case 16: HGRN2_LAUNCH(ST, 16, 1); break;           \
+      case 32: HGRN2_LAUNCH(ST, 32, 2); break;           \
+      case 64: HGRN2_LAUNCH(ST, 64, 4); break;           \
+      case 128: HGRN2_LAUNCH(ST, 128, 4); break;         \
+      default: HGRN2_LAUNCH(ST, 0, 1); break;            \
+    }                                                    \
   } while (0)
   if (dt == 0) HGRN2_BY_D(u16);
   else if (dt == 1) HGRN2_BY_D(float);

@@ -61,11 +61,12 @@ __device__ __forceinline__ float group4_sum(float v) {
   return v + __shfl_xor(v, 32, 64);
 }
 
+template <bool WIDE>
 __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int H = a.H, G = a.G, dq = a.dq, dv = a.dv, Hp = a.Hp, CG = a.CG;
   const int ldk = dq + 8;                         // padded K row (elements)
-  const bool wide = a.wide != 0;
+  constexpr bool wide = WIDE;
   const int dvw = wide ? 512 : 128;               // value slice of a workgroup
   const int dvo = (blockIdx.z % a.ndvs) * dvw;
   const int hbase = ((blockIdx.z / a.ndvs) % a.nhs) * NW;
@@ -464,11 +465,19 @@ extern "C" int dli_window_attention_mfma(
   const size_t sh = fixed + CG * per_cg;
   static bool raised = false;
   if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)window_attention_mfma_kernel,
+    hipError_t e = hipFuncSetAttribute((const void*)window_attention_mfma_kernel<false>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)window_attention_mfma_kernel<true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) return (int)e;
     raised = true;
   }
+#define WA_LAUNCH(GRID)                                                           \
+  do {                                                                            \
+    if (wide) window_attention_mfma_kernel<true><<<GRID, 512, sh, st>>>(a);       \
+    else window_attention_mfma_kernel<false><<<GRID, 512, sh, st>>>(a);           \
+  } while (0)
   const int ndvs = (dv + dvw - 1) / dvw, qtiles = (max_seqlen + TQ - 1) / TQ;
   const int nhs = wide ? (H + NW - 1) / NW : 1;
   const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, H, dv, window, wide) : 1;
@@ -478,7 +487,7 @@ extern "C" int dli_window_attention_mfma(
              nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);
-    window_attention_mfma_kernel<<<grid, 512, sh, st>>>(a);
+    WA_LAUNCH(grid);
     DLI_RETURN_LAUNCH();
   }
   if (T <= 0 || (H * dv) % 4 || ldo % 4) return (int)hipErrorInvalidValue;
@@ -488,10 +497,10 @@ extern "C" int dli_window_attention_mfma(
   a.o_ws_stride = (long)T * H * dv;
   a.mode = 1;
   a.ndvs = 1;                                     // the statistics do not depend on the slice
-  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, nhs * nsplit), 512, sh, st>>>(a);
+  WA_LAUNCH(dim3(qtiles, num_seqs, nhs * nsplit));
   a.mode = 2;
   a.ndvs = ndvs;
-  window_attention_mfma_kernel<<<dim3(qtiles, num_seqs, ndvs * nhs * nsplit), 512, sh, st>>>(a);
+  WA_LAUNCH(dim3(qtiles, num_seqs, ndvs * nhs * nsplit));
   const long quads = (long)T * (H * dv / 4);
   split_reduce_kernel<<<(int)((quads + 255) / 256), 256, 0, st>>>(
       (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv);
