@@ -47,6 +47,10 @@ struct MfmaArgs {
   // one per wave, and the wave's 32 accumulator blocks cover a 512-wide value slice instead
   // of 4 heads x 128 — latent attention's 512-wide values without recomputing the scores
   int wide, nhs;
+  // rows-are-heads form of a decode step whose heads all share one cached row per position
+  // (latent attention): the launcher presents token t's H heads as H query rows of a
+  // one-head problem, all at token t's position: rowmul = H (cu and positions are per token)
+  int rowmul;
   float* stats_ws;   // [S][q tiles][nsplit][H][TQ][2]
   float* o_ws;       // [nsplit][T][H*dv]
   long o_ws_stride;  // T * H * dv
@@ -83,17 +87,17 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
   const int s = blockIdx.y;
-  const int t0 = a.cu[s] + blockIdx.x * TQ;
-  const int t_end = a.cu[s + 1];
+  const int t0 = a.cu[s] * a.rowmul + blockIdx.x * TQ;
+  const int t_end = a.cu[s + 1] * a.rowmul;
   if (t0 >= t_end) return;
   const int nq = min(TQ, t_end - t0);
-  const int p0 = a.positions[t0];                 // positions of a portion are consecutive
-  const int p_last = p0 + nq - 1;
+  const int p0 = a.positions[t0 / a.rowmul];      // positions of a portion are consecutive
+  const int p_last = a.rowmul > 1 ? p0 : p0 + nq - 1;
   const int lo = max(0, p0 - a.window + 1);
   const int ntiles = (p_last - lo) / TK + 1;
   const int* bt = a.block_tables + (long)s * a.bt_stride;
   const int hpg = H / G;
-  const int my_p = p0 + fr;                       // this lane's query position (column fr)
+  const int my_p = a.rowmul > 1 ? p0 : p0 + fr;   // this lane's query position (column fr)
   const bool my_q = fr < nq;
   const bool has_talk = a.talk != nullptr;
   const int Hp16 = (H + 15) & ~15;
@@ -427,7 +431,12 @@ static int pick_splits(int num_seqs, int max_seqlen, int H, int dv, int window, 
 
 extern "C" long dli_window_attention_mfma_workspace_bytes(int num_seqs, int max_seqlen, int T,
                                                           int H, int dv, int window,
-                                                          int mixing) {
+                                                          int mixing, int rowhead) {
+  if (rowhead) {
+    max_seqlen = H;
+    T *= H;
+    H = 1;
+  }
   const int nsplit = pick_splits(num_seqs, max_seqlen, H, dv, window, mixing == 0);
   if (nsplit == 1) return 0;
   const long qtiles = (max_seqlen + TQ - 1) / TQ;
@@ -441,8 +450,20 @@ extern "C" int dli_window_attention_mfma(
     int ldo, const float* gate, int ldg, const float* slopes, const float* talk, const int* cu,
     const int* positions, const int* block_tables, int bt_stride, int block_size, int num_seqs,
     int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int T, void* ws,
-    hipStream_t st) {
+    int rowhead, hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
+  int rowmul = 1;
+  if (rowhead) {
+    if (talk != nullptr || gate != nullptr || slopes != nullptr || G != 1 || max_seqlen != 1 ||
+        ldq != H * dq || ldo != H * dv)
+      return (int)hipErrorInvalidValue;
+    rowmul = H;            // token t's heads = rows [t*H, (t+1)*H) of a one-head problem
+    max_seqlen = H;
+    T *= H;
+    ldq = dq;
+    ldo = dv;
+    H = 1;
+  }
   const bool aligned = (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 &&
                        (uintptr_t)out % 8 == 0 && ldq % 8 == 0 && k_stride % 8 == 0 &&
                        v_stride % 8 == 0 && ldo % 4 == 0;
@@ -483,7 +504,7 @@ extern "C" int dli_window_attention_mfma(
   const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, H, dv, window, wide) : 1;
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
-             H, G, dq, dv, window, scale, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs,
+             H, G, dq, dv, window, scale, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
              nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);

@@ -82,8 +82,8 @@ _SIGS = {
     "dli_window_attention": [P, I, P, L, P, L, P, I, P, I, P, P, P, P, P,
                              I, I, I, I, I, I, I, I, I, F, I, P],
     "dli_window_attention_mfma": [P, I, P, L, P, L, P, I, P, I, P, P, P, P, P,
-                                  I, I, I, I, I, I, I, I, I, F, I, P, P],
-    "dli_window_attention_mfma_workspace_bytes": [I, I, I, I, I, I, I],
+                                  I, I, I, I, I, I, I, I, I, F, I, P, I, P],
+    "dli_window_attention_mfma_workspace_bytes": [I, I, I, I, I, I, I, I],
     "dli_hgrn2": [P, I, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
 }
 

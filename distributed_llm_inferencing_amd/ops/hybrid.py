@@ -198,15 +198,20 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
     if q.dtype == torch.bfloat16 and MFMA_ATTENTION:
         # the MFMA form; shapes it does not take (odd head sizes, > 32 heads) fall through
         lib = N.require_native()
+        # decode steps of heads that share one cached row per position (latent attention):
+        # the heads become the query rows of a one-head problem
+        rowhead = int(G == 1 and H > 1 and int(max_seqlen) == 1 and talk is None and gate is None
+                      and slopes is None and q.stride(0) == H * dq)
         nb = lib.dli_window_attention_mfma_workspace_bytes(S, int(max_seqlen), T, H, dv,
-                                                           int(window), int(talk is not None))
+                                                           int(window), int(talk is not None),
+                                                           rowhead)
         ws = _gemm.workspace(q.device, nb) if nb else None       # key-split form (decode steps)
         rc = lib.dli_window_attention_mfma(
             _p(q), q.stride(0), _p(k_cache), k_cache.stride(0), _p(v_cache), v_cache.stride(0),
             _p(out), out.stride(0), _p(gate), gate.stride(0) if gate is not None else 0,
             _p(slopes), _p(talk), _p(cu_seqlens), _p(positions), _p(block_tables),
             block_tables.stride(0), block_size, S, int(max_seqlen), H, G, dq, dv, int(window),
-            float(scale), T, _p(ws), _st())
+            float(scale), T, _p(ws), rowhead, _st())
         if rc == 0:
             return out
         if rc != _NOT_SUPPORTED:

@@ -392,6 +392,25 @@ def test_mfma_window_attention_matches_reference(gpu, H, G, dq, dv, win, talk, s
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,dq,dv,win", [(32, 96, 64, 300), (5, 64, 32, 40), (16, 160, 144, 1000)])
+def test_mfma_decode_rows_of_shared_kv_heads(gpu, H, dq, dv, win):
+    """Decode steps (one token a sequence) of heads that share one cached row per position,
+    values = the row's first columns: the kernel's rows-are-heads form, with key splits."""
+    from distributed_llm_inferencing_amd.ops import hybrid as Hy
+    from distributed_llm_inferencing_amd.ops import reference as R
+    starts = [0, 700, 31, 299, 300, 1, 64]
+    lens = [1] * len(starts)
+    q, kc, _, cu, pos, bt = _paged_case(lens, starts, H, 1, dq, dv, 16, True, seed=H)
+    scale = dq ** -0.5
+    want = R.window_attention(q, kc, kc, dq, dv, H, 1, cu, pos, bt, 16, win, scale,
+                              out_dtype=torch.float32)
+    d = lambda t: t.to(gpu)      # noqa: E731
+    got = Hy.window_attention(d(q), d(kc), d(kc), dq, dv, H, 1, d(cu), 1, d(pos), d(bt), 16, win,
+                              scale).float().cpu()
+    assert (got - want).abs().max() < 0.03 * want.abs().max().item() + 0.02
+
+
+@pytest.mark.gpu
 def test_model_on_mfma_sized_heads(gpu):
     """A whole model whose head sizes take the MFMA attention path, cut in portions."""
     c = config([attn(heads=4, kv=2, dim=32, win=20, ff=64), hgrn(heads=2, dim=16, vdim=32),
