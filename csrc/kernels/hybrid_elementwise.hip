@@ -48,22 +48,40 @@ template <typename S>
 __global__ void __launch_bounds__(256) resadd_groupnorm_kernel(
     float* __restrict__ x, const float* __restrict__ y, int ldy, const S* __restrict__ bias,
     float keep, float mult, const S* __restrict__ w, S* __restrict__ h, int ldh, int dim,
-    int groups, float eps, const long* __restrict__ rows_idx) {
-  extern __shared__ float row[];            // dim floats + groups partial sums
+    int groups, float eps, const long* __restrict__ rows_idx, bool vec4) {
+  extern __shared__ __attribute__((aligned(16))) float row[];   // dim floats + group scales
   float* gsum = row + dim;
   const int r = blockIdx.x;
   const long src = rows_idx ? rows_idx[r] : r;
   float* xr = x + src * dim;
   for (int g = threadIdx.x; g < groups; g += blockDim.x) gsum[g] = 0.f;
-  for (int c = threadIdx.x; c < dim; c += blockDim.x) {
-    float v = xr[c];
-    if (rows_idx == nullptr) {
-      v = keep != 0.f ? v * keep : 0.f;
-      if (y != nullptr) v += mult * y[(long)r * ldy + c];
-      if (bias != nullptr) v += ldf(bias + c);
-      if (y != nullptr || bias != nullptr || keep != 1.f) xr[c] = v;
+  const bool update = rows_idx == nullptr && (y != nullptr || bias != nullptr || keep != 1.f);
+  if (vec4) {                               // 16-byte loads and stores of the fp32 rows
+    for (int c = threadIdx.x * 4; c < dim; c += blockDim.x * 4) {
+      f32x4 v = *reinterpret_cast<const f32x4*>(xr + c);
+      if (rows_idx == nullptr) {
+        if (keep == 0.f) v = f32x4{0.f, 0.f, 0.f, 0.f};
+        else if (keep != 1.f) v *= keep;
+        if (y != nullptr) v += mult * *reinterpret_cast<const f32x4*>(y + (long)r * ldy + c);
+        if (bias != nullptr) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) v[u] += ldf(bias + c + u);
+        }
+        if (update) *reinterpret_cast<f32x4*>(xr + c) = v;
+      }
+      *reinterpret_cast<f32x4*>(row + c) = v;
     }
-    row[c] = v;
+  } else {
+    for (int c = threadIdx.x; c < dim; c += blockDim.x) {
+      float v = xr[c];
+      if (rows_idx == nullptr) {
+        v = keep != 0.f ? v * keep : 0.f;
+        if (y != nullptr) v += mult * y[(long)r * ldy + c];
+        if (bias != nullptr) v += ldf(bias + c);
+        if (update) xr[c] = v;
+      }
+      row[c] = v;
+    }
   }
   __syncthreads();
   if (h == nullptr) return;
@@ -103,6 +121,21 @@ __global__ void __launch_bounds__(256) gelu_mul_kernel(
   const int t = (int)(gid / F), c = (int)(gid % F);
   const float* r = gu + (long)t * ldg;
   stf(out + (long)t * ldo + c, gelu_tanh32(r[c]) * r[F + c]);
+}
+
+// 4 features a thread (F, ldg multiples of 4, 16-byte aligned rows): 16-byte loads
+template <typename S>
+__global__ void __launch_bounds__(256) gelu_mul4_kernel(
+    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F) {
+  const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int f4 = F >> 2;
+  if (gid >= (long)T * f4) return;
+  const int t = (int)(gid / f4), c = (int)(gid % f4) * 4;
+  const float* r = gu + (long)t * ldg;
+  const f32x4 g = *reinterpret_cast<const f32x4*>(r + c);
+  const f32x4 u = *reinterpret_cast<const f32x4*>(r + F + c);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) stf(out + (long)t * ldo + c + i, gelu_tanh32(g[i]) * u[i]);
 }
 
 // proj row: [H*d q | G*d k | ...]; one wave per (token, head) unit, H + G units per token.
@@ -218,13 +251,15 @@ extern "C" int dli_resadd_groupnorm(float* x, const float* y, int ldy, const voi
   if (groups < 1 || dim % groups || (size_t)(dim + groups) * 4 > 60000)
     return (int)hipErrorInvalidValue;
   const size_t sh = (size_t)(dim + groups) * 4;
+  const bool vec4 = dim % 4 == 0 && (uintptr_t)x % 16 == 0 &&
+                    (y == nullptr || ((uintptr_t)y % 16 == 0 && ldy % 4 == 0));
   DT_SWITCH(dt,
             (resadd_groupnorm_kernel<u16><<<rows, 256, sh, st>>>(
                 x, y, ldy, (const u16*)bias, keep, mult, (const u16*)w, (u16*)h, ldh, dim, groups,
-                eps, rows_idx)),
+                eps, rows_idx, vec4)),
             (resadd_groupnorm_kernel<float><<<rows, 256, sh, st>>>(
                 x, y, ldy, (const float*)bias, keep, mult, (const float*)w, (float*)h, ldh, dim,
-                groups, eps, rows_idx)));
+                groups, eps, rows_idx, vec4)));
   DLI_RETURN_LAUNCH();
 }
 
@@ -240,6 +275,12 @@ extern "C" int dli_concat_cast(void* out, const float* a, const float* b, int T,
 extern "C" int dli_gelu_mul(void* out, int ldo, const float* gu, int ldg, int T, int F, int dt,
                             hipStream_t st) {
   if (T <= 0) return 0;
+  if (F % 4 == 0 && ldg % 4 == 0 && (uintptr_t)gu % 16 == 0) {
+    const int nb4 = (int)(((long)T * (F / 4) + 255) / 256);
+    DT_SWITCH(dt, (gelu_mul4_kernel<u16><<<nb4, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F)),
+              (gelu_mul4_kernel<float><<<nb4, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F)));
+    DLI_RETURN_LAUNCH();
+  }
   const int nb = (int)(((long)T * F + 255) / 256);
   DT_SWITCH(dt, (gelu_mul_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F)),
             (gelu_mul_kernel<float><<<nb, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F)));
