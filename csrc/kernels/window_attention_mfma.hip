@@ -23,7 +23,8 @@
 
 namespace {
 
-constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8, STG = 4;
+constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8, STG = 2;
+constexpr float LOG2E = 1.4426950408889634f;
 
 struct MfmaArgs {
   const u16* q; int ldq;
@@ -51,6 +52,9 @@ struct MfmaArgs {
   // (latent attention): the launcher presents token t's H heads as H query rows of a
   // one-head problem, all at token t's position: rowmul = H (cu and positions are per token)
   int rowmul;
+  // > 0: the cache rows of the whole window (slot_cap ints) are looked up once at kernel start
+  // instead of per key tile (one global round trip and one barrier less per tile)
+  int slot_cap;
   float* stats_ws;   // [S][q tiles][nsplit][H][TQ][2]
   float* o_ws;       // [nsplit][T][H*dv]
   long o_ws_stride;  // T * H * dv
@@ -69,7 +73,8 @@ template <bool WIDE>
 __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int H = a.H, G = a.G, dq = a.dq, dv = a.dv, Hp = a.Hp, CG = a.CG;
-  const int ldk = dq + 8;                         // padded K row (elements)
+  const int ldk = dq + 16;                        // padded K row (elements): 8 extra dwords
+  const int HpS = Hp + 8;                         // padded row of the mix operand
   constexpr bool wide = WIDE;
   const int dvw = wide ? 512 : 128;               // value slice of a workgroup
   const int dvo = (blockIdx.z % a.ndvs) * dvw;
@@ -77,12 +82,14 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   const int split = blockIdx.z / (a.ndvs * a.nhs);
   const int dvc = min(dvw, dv - dvo);
   const int dvb = dvc >> 4;
+  // the K tiles (score phase) and the transposed V tiles (apply phase) of a key tile are never
+  // live together: one region serves both, so every kv head of the tile is staged at once
   u16* Ks = (u16*)smem;                           // [CG][TK][ldk]
-  u16* Vt = Ks + CG * TK * ldk;                   // [CG][dvw][40]
-  u16* Pm = Vt + CG * dvw * 40;                   // [TQ*TK][Hp]
-  u16* Pp = Pm + (wide ? 0 : TQ * TK * Hp);       // [H][TQ][40] (wide: [NW][TQ][40], by wave)
+  u16* Vt = Ks;                                   // [CG][dvw][40]
+  u16* Pm = Ks + CG * max(TK * ldk, dvw * 40);    // [TQ*TK][Hp]
+  u16* Pp = Pm + (wide ? 0 : TQ * TK * HpS);      // [H][TQ][40] (wide: [NW][TQ][40], by wave)
   u16* Tk = Pp + (wide ? NW : H) * TQ * 40;       // [Hp16][Hp] talk in bf16, zero padded
-  int* slot = (int*)(Tk + (wide ? 0 : ((H + 15) & ~15) * Hp));   // [TK]
+  int* slot_all = (int*)(Tk + (wide ? 0 : ((H + 15) & ~15) * Hp));   // [TK] or [slot_cap]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
@@ -110,7 +117,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   }
   // zero the mix operand once: head columns [H, Hp) stay zero for the whole kernel
   if (has_talk)
-    for (int i = tid; i < TQ * TK * Hp / 2; i += 512) ((uint32_t*)Pm)[i] = 0u;
+    for (int i = tid; i < TQ * TK * HpS / 2; i += 512) ((uint32_t*)Pm)[i] = 0u;
 
   float m_run[MAXHW], l_run[MAXHW];
   f32x4 oacc[MAXHW][MAXDVB];
@@ -122,6 +129,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
     for (int b = 0; b < MAXDVB; ++b) oacc[hh][b] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int nf = dq >> 5;                         // 32-wide K-steps of the score product
+  const float scale2 = a.scale * LOG2E;
   int tile_lo = 0, tile_hi = ntiles;
   if (a.nsplit > 1) {
     const int per = (ntiles + a.nsplit - 1) / a.nsplit;
@@ -140,50 +148,87 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
       float L = 0.f;
       for (int k2 = 0; k2 < a.nsplit; ++k2) {
         const float* pr = a.stats_ws + (((stats_base + k2) * H + h) * TQ + fr) * 2;
-        if (pr[0] != -INFINITY) L += pr[1] * expf(pr[0] - M);
+        if (pr[0] != -INFINITY) L += pr[1] * __builtin_amdgcn_exp2f(pr[0] - M);
       }
       m_run[hh] = M;
       l_run[hh] = L;
     }
   }
   const int pass_lo = a.mode == 2 ? 1 : 0, pass_hi = a.mode == 1 ? 1 : 2;
+  // staging walks: per-thread start indices and 512-chunk strides, divided once
+  const int kcpr = dq >> 3, vcpr = dvc >> 3;
+  const int krow0 = tid / kcpr, kch0 = tid % kcpr, kq512 = 512 / kcpr, kr512 = 512 % kcpr;
+  const int vrest0 = tid >> 5, vc0 = vrest0 / vcpr, vch0 = vrest0 % vcpr;
+  const int vq16 = 16 / vcpr, vr16 = 16 % vcpr;
+  uint4 qcur[4];                                  // prefetched query fragments of head qh
+  int qh = -1;
+  auto load_q = [&](int h, int f0, uint4* dst) {
+    const u16* qrow = a.q + (long)(t0 + fr) * a.ldq + (long)h * dq + fq * 8;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      dst[u] = uint4{0u, 0u, 0u, 0u};
+      if (my_q && f0 + u < nf) dst[u] = *reinterpret_cast<const uint4*>(qrow + (f0 + u) * 32);
+    }
+  };
+  const bool slots_once = a.slot_cap >= ntiles * TK;
+  if (slots_once) {
+    for (int i = tid + tile_lo * TK; i < tile_hi * TK; i += 512) {
+      const int j = lo + i;
+      slot_all[i] = j <= p_last ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
+    }
+  }
 
   for (int pass = pass_lo; pass < pass_hi; ++pass) {
     for (int tile = tile_lo; tile < tile_hi; ++tile) {
       const int j0 = lo + tile * TK;
-      __syncthreads();                            // previous tile's readers are done
-      if (tid < TK) {
-        const int j = j0 + tid;
-        slot[tid] = j <= p_last ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
+      int* slot = slots_once ? slot_all + tile * TK : slot_all;
+      if (!slots_once) {
+        __syncthreads();                          // previous tile's readers are done
+        if (tid < TK) {
+          const int j = j0 + tid;
+          slot[tid] = j <= p_last ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
+        }
       }
       for (int c0 = 0; c0 < G; c0 += CG) {
         const int cg = min(CG, G - c0);
+        {                                         // this wave's first head of the step: its
+          int h0 = -1;                            // query fragments fly with the K tiles
+#pragma unroll
+          for (int h2 = MAXHW - 1; h2 >= 0; --h2) {
+            const int hc = wide ? hbase + wave : wave + h2 * NW;
+            if ((!wide || h2 == 0) && hc < H && hc / hpg >= c0 && hc / hpg < c0 + cg) h0 = hc;
+          }
+          qh = h0;
+          if (h0 >= 0) load_q(h0, 0, qcur);
+        }
         __syncthreads();                          // slot table ready; Ks free
         {                                         // stage K tiles of kv heads [c0, c0+cg)
-          const int cpr = dq >> 3;                // 16-byte chunks per row
-          const int total = cg * TK * cpr;
+          // chunk i = (c * TK + r) * kcpr + ch; a thread's chunks are 512 apart, walked by
+          // increments (no division in the loop)
+          const int total = cg * TK * kcpr;
+          int row = krow0, ch = kch0;
           for (int base = 0; base < total; base += 512 * STG) {
             uint4 val[STG];                       // STG loads in flight per thread
+            int lds_off[STG];
 #pragma unroll
             for (int u = 0; u < STG; ++u) {
-              const int i = base + u * 512 + tid;
               val[u] = uint4{0u, 0u, 0u, 0u};
-              if (i < total) {
-                const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
+              lds_off[u] = -1;
+              if (base + u * 512 + tid < total) {
+                const int c = row >> 5, r = row & (TK - 1);
+                lds_off[u] = row * ldk + ch * 8;
                 const int sl = slot[r];
                 if (sl >= 0)
                   val[u] = *reinterpret_cast<const uint4*>(a.k + (long)sl * a.k_stride +
-                                                           (long)(c0 + c) * dq + ch * 8);
+                                                           (c0 + c) * dq + ch * 8);
               }
+              row += kq512;
+              ch += kr512;
+              if (ch >= kcpr) { ch -= kcpr; row += 1; }
             }
 #pragma unroll
-            for (int u = 0; u < STG; ++u) {
-              const int i = base + u * 512 + tid;
-              if (i < total) {
-                const int c = i / (TK * cpr), r = (i / cpr) % TK, ch = i % cpr;
-                *reinterpret_cast<uint4*>(Ks + ((long)c * TK + r) * ldk + ch * 8) = val[u];
-              }
-            }
+            for (int u = 0; u < STG; ++u)
+              if (lds_off[u] >= 0) *reinterpret_cast<uint4*>(Ks + lds_off[u]) = val[u];
           }
         }
         __syncthreads();
@@ -195,18 +240,24 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
           if (c < c0 || c >= c0 + cg) continue;
           const u16* kt = Ks + (long)(c - c0) * TK * ldk;
           f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
-          const u16* qrow = a.q + (long)(t0 + fr) * a.ldq + (long)h * dq + fq * 8;
-          for (int f0 = 0; f0 < nf; f0 += 4) {     // 4 query fragments in flight
-            uint4 qv[4];
+          // query fragments, 4 at a time, one group ahead: the next group (of this head, or
+          // the first of this wave's next head) is requested before this group's MFMAs
+          int hn = -1;                            // this wave's next head of the step
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              qv[u] = uint4{0u, 0u, 0u, 0u};
-              if (my_q && f0 + u < nf) qv[u] = *reinterpret_cast<const uint4*>(qrow + (f0 + u) * 32);
+          for (int h2 = MAXHW - 1; h2 > hh; --h2) {
+            const int hc = wave + h2 * NW;
+            if (!wide && hc < H && hc / hpg >= c0 && hc / hpg < c0 + cg) hn = hc;
+          }
+          if (qh != h) load_q(h, 0, qcur);        // not prefetched (first head of the step)
+          for (int f0 = 0; f0 < nf; f0 += 4) {
+            uint4 qnxt[4];
+            if constexpr (wide) {                 // registers allow the look-ahead only here
+              if (f0 + 4 < nf) load_q(h, f0 + 4, qnxt);
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
               if (f0 + u >= nf) continue;
-              const bf16x8 qf = *reinterpret_cast<const bf16x8*>(&qv[u]);
+              const bf16x8 qf = *reinterpret_cast<const bf16x8*>(&qcur[u]);
 #pragma unroll
               for (int kb = 0; kb < 2; ++kb) {
                 const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
@@ -214,44 +265,71 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
                 sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf, sacc[kb], 0, 0, 0);
               }
             }
+            if constexpr (wide) {
+#pragma unroll
+              for (int u = 0; u < 4; ++u) qcur[u] = qnxt[u];
+            } else {
+              if (f0 + 4 < nf) load_q(h, f0 + 4, qcur);
+              else if (hn >= 0) load_q(hn, 0, qcur);   // next head's first group, under the
+            }                                          // softmax arithmetic of this one
           }
-          // lane: query fr, keys j0 + kb*16 + 4*fq + r
-          const float slope = a.slopes ? a.slopes[h] : 0.f;
+          qh = hn;
+          // lane: query fr, keys j0 + kb*16 + 4*fq + r. Scores are kept in the log2 domain
+          // (scale and slope carry log2 e), so every exponential is one v_exp_f32:
+          //   x = s * scale2 - slope2 * (p - j) = fma(s, scale2, slope2 * (j - p))
+          const float slope2 = a.slopes ? a.slopes[h] * LOG2E : 0.f;
+          const float b0 = slope2 * (float)(j0 + fq * 4 - my_p);
           float sv[8];
           float tmax = -INFINITY;
+          // interior tiles (every key visible to every query row): no masking arithmetic
+          const bool interior = nq == TQ && j0 + TK - 1 <= p0 && j0 > p_last - a.window;
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int j = j0 + kb * 16 + fq * 4 + r;
-              const int dist = my_p - j;
-              float x = sacc[kb][r] * a.scale - slope * (float)dist;
-              if (!my_q || dist < 0 || dist >= a.window) x = -INFINITY;
+              float x = fmaf(sacc[kb][r], scale2, b0 + slope2 * (float)(kb * 16 + r));
+              if (!interior) {
+                const int dist = my_p - (j0 + kb * 16 + fq * 4 + r);
+                if (!my_q || dist < 0 || dist >= a.window) x = -INFINITY;
+              }
               sv[kb * 4 + r] = x;
               tmax = fmaxf(tmax, x);
             }
           if (pass == 0) {
             tmax = group4_max(tmax);
             const float m_new = fmaxf(m_run[hh], tmax);
+            // exp2(-inf - m) = 0 for a finite m; a row with no visible key yet keeps m = -inf
+            const float mm = m_new == -INFINITY ? 0.f : m_new;
             float sum = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) sum += sv[i] == -INFINITY ? 0.f : expf(sv[i] - m_new);
+            for (int i = 0; i < 8; ++i) sum += __builtin_amdgcn_exp2f(sv[i] - mm);
             sum = group4_sum(sum);
-            const float carry = m_run[hh] == -INFINITY ? 0.f : l_run[hh] * expf(m_run[hh] - m_new);
-            l_run[hh] = carry + sum;
+            l_run[hh] = l_run[hh] * __builtin_amdgcn_exp2f(m_run[hh] - mm) + sum;
             m_run[hh] = m_new;
           } else {
             const float inv = l_run[hh] > 0.f ? 1.f / l_run[hh] : 0.f;
+            const float mm = m_run[hh] == -INFINITY ? 0.f : m_run[hh];
+            float w[8];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int i = 0; i < 8; ++i) w[i] = __builtin_amdgcn_exp2f(sv[i] - mm) * inv;
+            if (has_talk) {
+              // row = key * TQ + query: the 16 queries of a key sit 20 dwords apart
+              u16* dst = Pm + (fq * 4 * TQ + fr) * HpS + h;
 #pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                const float x = sv[kb * 4 + r];
-                const float w = x == -INFINITY ? 0.f : expf(x - m_run[hh]) * inv;
-                const int key = kb * 16 + fq * 4 + r;
-                if (has_talk) Pm[(long)(fr * TK + key) * Hp + h] = f2bf(w);
-                else Pp[((long)(wide ? wave : h) * TQ + fr) * 40 + key] = f2bf(w);
+              for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dst[(kb * 16 + r) * TQ * HpS] = f2bf(w[kb * 4 + r]);
+            } else {
+              // 4 consecutive keys of one query: one 8-byte store per key block
+              u16* dst = Pp + ((wide ? wave : h) * TQ + fr) * 40 + fq * 4;
+#pragma unroll
+              for (int kb = 0; kb < 2; ++kb) {
+                uint2 pk;
+                pk.x = pack2bf(w[kb * 4], w[kb * 4 + 1]);
+                pk.y = pack2bf(w[kb * 4 + 2], w[kb * 4 + 3]);
+                *reinterpret_cast<uint2*>(dst + kb * 16) = pk;
               }
+            }
           }
         }
       }
@@ -267,11 +345,11 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
             const bf16x8 tf = *reinterpret_cast<const bf16x8*>(
                 Tk + (long)(hb * 16 + fr) * Hp + kk + fq * 8);
             const bf16x8 pf = *reinterpret_cast<const bf16x8*>(
-                Pm + (long)(xb * 16 + fr) * Hp + kk + fq * 8);
+                Pm + (long)(xb * 16 + fr) * HpS + kk + fq * 8);
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf, pf, acc, 0, 0, 0);
           }
-          // lane: heads hb*16 + 4*fq + r, x = xb*16 + fr  (x = query * TK + key)
-          const int x = xb * 16 + fr, qi = x / TK, key = x % TK;
+          // lane: heads hb*16 + 4*fq + r, x = xb*16 + fr  (x = key * TQ + query)
+          const int x = xb * 16 + fr, qi = x % TQ, key = x / TQ;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int h = hb * 16 + fq * 4 + r;
@@ -284,31 +362,34 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         const int cg = min(CG, G - c0);
         __syncthreads();                          // Pp complete (first step) / Vt free
         {
-          const int cpr = dvc >> 3;
-          const int total = cg * TK * cpr;
+          // chunk i = (c * vcpr + ch) * TK + r: consecutive threads take consecutive keys of one
+          // 8-dim chunk, so their transposed 2-byte stores fall into consecutive LDS addresses
+          const int total = cg * TK * vcpr;
+          const int r = tid & (TK - 1);
+          int cc = vc0, ch = vch0;
           for (int base = 0; base < total; base += 512 * STG) {
             uint4 val[STG];
+            int lds_off[STG];
 #pragma unroll
             for (int u = 0; u < STG; ++u) {
-              const int i = base + u * 512 + tid;
               val[u] = uint4{0u, 0u, 0u, 0u};
-              if (i < total) {
-                // consecutive threads take consecutive keys of one 8-dim chunk: their
-                // transposed 2-byte stores then fall into consecutive LDS addresses
-                const int r = i % TK, ch = (i / TK) % cpr, c = i / (TK * cpr);
+              lds_off[u] = -1;
+              if (base + u * 512 + tid < total) {
+                lds_off[u] = (cc * dvw + ch * 8) * 40 + r;
                 const int sl = slot[r];
                 if (sl >= 0)
                   val[u] = *reinterpret_cast<const uint4*>(a.v + (long)sl * a.v_stride +
-                                                           (long)(c0 + c) * dv + dvo + ch * 8);
+                                                           (c0 + cc) * dv + dvo + ch * 8);
               }
+              cc += vq16;
+              ch += vr16;
+              if (ch >= vcpr) { ch -= vcpr; cc += 1; }
             }
 #pragma unroll
             for (int u = 0; u < STG; ++u) {
-              const int i = base + u * 512 + tid;
-              if (i < total) {
-                const int r = i % TK, ch = (i / TK) % cpr, c = i / (TK * cpr);
+              if (lds_off[u] >= 0) {
                 const u16* e = reinterpret_cast<const u16*>(&val[u]);
-                u16* dst = Vt + ((long)c * dvw + ch * 8) * 40 + r;
+                u16* dst = Vt + lds_off[u];
 #pragma unroll
                 for (int w = 0; w < 8; ++w) dst[w * 40] = e[w];
               }
@@ -473,12 +554,15 @@ extern "C" int dli_window_attention_mfma(
     return (int)hipErrorNotSupported;
   const int dvw = wide ? 512 : 128;
   const int Hp = (H + 31) & ~31, Hp16 = (H + 15) & ~15;
-  const int ldk = dq + 8;
+  const int ldk = dq + 16;
+  // the whole window's cache rows in LDS when they take at most 16 KB
+  int slot_cap = ((window + TQ - 2) / TK + 2) * TK;
+  if ((size_t)slot_cap * 4 > 16 * 1024) slot_cap = 0;
   const size_t fixed = (wide ? (size_t)NW * TQ * 40
-                             : (size_t)TQ * TK * Hp + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
-                       TK * 4 + 64;
-  const size_t per_cg = ((size_t)TK * ldk + (size_t)dvw * 40) * 2;
-  const size_t budget = 150 * 1024;
+                             : (size_t)TQ * TK * (Hp + 8) + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
+                       (size_t)(slot_cap > TK ? slot_cap : TK) * 4 + 64;
+  const size_t per_cg = (size_t)((TK * ldk > dvw * 40) ? TK * ldk : dvw * 40) * 2;
+  const size_t budget = 158 * 1024;
   if (fixed + per_cg > budget) return (int)hipErrorNotSupported;
   int CG = (int)((budget - fixed) / per_cg);
   CG = CG > G ? G : CG;
@@ -505,7 +589,7 @@ extern "C" int dli_window_attention_mfma(
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
              H, G, dq, dv, window, scale, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
-             nullptr, nullptr, 0};
+             slot_cap, nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);
     WA_LAUNCH(grid);
