@@ -23,7 +23,7 @@
 
 namespace {
 
-constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8, STG = 2;
+constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8;
 constexpr float LOG2E = 1.4426950408889634f;
 
 struct MfmaArgs {
@@ -76,6 +76,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   const int ldk = dq + 16;                        // padded K row (elements): 8 extra dwords
   const int HpS = Hp + 8;                         // padded row of the mix operand
   constexpr bool wide = WIDE;
+  // 16-byte staging loads in flight per thread: what the register budget of the form allows
+  constexpr int STG = WIDE ? 5 : 2;
   const int dvw = wide ? 512 : 128;               // value slice of a workgroup
   const int dvo = (blockIdx.z % a.ndvs) * dvw;
   const int hbase = ((blockIdx.z / a.ndvs) % a.nhs) * NW;
