@@ -135,7 +135,8 @@ def test_group_norm_and_gated_ff_ops(device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("shape", [(7, 33, 50), (70, 130, 96), (3, 64, 128), (129, 20, 8)])
+@pytest.mark.parametrize("shape", [(7, 33, 50), (70, 130, 96), (3, 64, 128), (129, 20, 8),
+                                   (70, 33, 128), (5, 509, 64), (300, 81, 192), (1, 7, 256)])
 def test_linear_any_shapes(shape, device, dtype):
     from distributed_llm_inferencing_amd.ops import hybrid as H
     M, N, K = shape
@@ -360,7 +361,8 @@ def _paged_case(lens, starts, H, G, dq, dv, block, shared_kv, seed, dtype=torch.
 @pytest.mark.parametrize("H,G,dq,dv,win,talk,shared", [
     (4, 2, 32, 32, 24, True, False), (8, 8, 64, 64, 100, True, False),
     (32, 8, 128, 128, 70, True, False), (5, 1, 96, 64, 33, False, True),
-    (16, 1, 160, 144, 64, False, True), (3, 3, 32, 32, 1, True, False)])
+    (16, 1, 160, 144, 64, False, True), (3, 3, 32, 32, 1, True, False),
+    (4, 2, 32, 48, 5000, True, False), (40, 5, 32, 32, 50, False, False)])
 def test_mfma_window_attention_matches_reference(gpu, H, G, dq, dv, win, talk, shared):
     from distributed_llm_inferencing_amd.ops import hybrid as Hy
     from distributed_llm_inferencing_amd.ops import reference as R
@@ -422,3 +424,25 @@ def test_model_on_mfma_sized_heads(gpu):
     eng = engine(c, w, "cuda", torch.bfloat16)
     close(replay(eng, t, [60]), want, torch.bfloat16, "whole")
     close(replay(eng, t, [17, 1, 1, 30, 2, 9]), want, torch.bfloat16, "portions")
+
+
+@pytest.mark.parametrize("device,dtype", CASES[:2])
+def test_generation_under_preemption(device, dtype):
+    """A pool too small for the batch: sequences are preempted (blocks and state slot given
+    back), re-admitted and recomputed from position 0; the tokens stay the oracle's."""
+    w = O.random_weights(FULL, seed=8, scale=1.5)
+    prompts = [toks(n, FULL["vocab"], 50 + n) for n in (14, 11, 16)]
+    new = 14
+    eng = engine(FULL, w, device, dtype, max_tokens=56, live=3)
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=new, do_sample=False,
+                                                ignore_eos=True))
+    assert eng.scheduler.num_preempted > 0
+    for p, o in zip(prompts, outs):
+        seq = list(p)
+        for tok in o.output_ids:
+            lg = O.forward(FULL, w, seq)[-1]
+            best = int(lg.argmax())
+            assert tok == best or (lg[best] - lg[tok]) / lg.std() < 1e-3
+            seq.append(tok)
+        assert len(o.output_ids) == new
+    assert eng.bm.num_free == eng.bm.num_blocks and eng.state_slots.num_free == 3
