@@ -21,6 +21,9 @@
 // tile's last query) get weight 0; a query row always sees itself, so l > 0.
 #include "common.h"
 
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void gbl_void;
+
 namespace {
 
 constexpr int TQ = 16, TK = 32, NW = 8, MAXHW = 4, MAXDVB = 8;
@@ -88,7 +91,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   // live together: one region serves both, so every kv head of the tile is staged at once
   u16* Ks = (u16*)smem;                           // [CG][TK][ldk]
   u16* Vt = Ks;                                   // [CG][dvw][40]
-  u16* Pm = Ks + CG * max(TK * ldk, dvw * 40);    // [TQ*TK][Hp]
+  u16* Pm = Ks + CG * max(TK * ldk, dvw * 40) + 512;   // [TQ*TK][Hp] (after 1 KiB of DMA slack)
   u16* Pp = Pm + (wide ? 0 : TQ * TK * HpS);      // [H][TQ][40] (wide: [NW][TQ][40], by wave)
   u16* Tk = Pp + (wide ? NW : H) * TQ * 40;       // [Hp16][Hp] talk in bf16, zero padded
   int* slot_all = (int*)(Tk + (wide ? 0 : ((H + 15) & ~15) * Hp));   // [TK] or [slot_cap]
@@ -158,8 +161,10 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   }
   const int pass_lo = a.mode == 2 ? 1 : 0, pass_hi = a.mode == 1 ? 1 : 2;
   // staging walks: per-thread start indices and 512-chunk strides, divided once
-  const int kcpr = dq >> 3, vcpr = dvc >> 3;
-  const int krow0 = tid / kcpr, kch0 = tid % kcpr, kq512 = 512 / kcpr, kr512 = 512 % kcpr;
+  const int vcpr = dvc >> 3;
+  const int rowB = ldk * 2;                       // bytes of a padded K row in LDS
+  const int drow0 = (wave * 1024 + lane * 16) / rowB, drem0 = (wave * 1024 + lane * 16) % rowB;
+  const int dq8k = (NW * 1024) / rowB, dr8k = (NW * 1024) % rowB;
   const int vrest0 = tid >> 5, vc0 = vrest0 / vcpr, vch0 = vrest0 % vcpr;
   const int vq16 = 16 / vcpr, vr16 = 16 % vcpr;
   uint4 qcur[4];                                  // prefetched query fragments of head qh
@@ -205,33 +210,26 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         }
         __syncthreads();                          // slot table ready; Ks free
         {                                         // stage K tiles of kv heads [c0, c0+cg)
-          // chunk i = (c * TK + r) * kcpr + ch; a thread's chunks are 512 apart, walked by
-          // increments (no division in the loop)
-          const int total = cg * TK * kcpr;
-          int row = krow0, ch = kch0;
-          for (int base = 0; base < total; base += 512 * STG) {
-            uint4 val[STG];                       // STG loads in flight per thread
-            int lds_off[STG];
-#pragma unroll
-            for (int u = 0; u < STG; ++u) {
-              val[u] = uint4{0u, 0u, 0u, 0u};
-              lds_off[u] = -1;
-              if (base + u * 512 + tid < total) {
-                const int c = row >> 5, r = row & (TK - 1);
-                lds_off[u] = row * ldk + ch * 8;
-                const int sl = slot[r];
-                if (sl >= 0)
-                  val[u] = *reinterpret_cast<const uint4*>(a.k + (long)sl * a.k_stride +
-                                                           (c0 + c) * dq + ch * 8);
-              }
-              row += kq512;
-              ch += kr512;
-              if (ch >= kcpr) { ch -= kcpr; row += 1; }
+          // LDS-DMA (global_load_lds_dwordx4): no staging registers, every piece in flight at
+          // once. A wave's instruction fills 1 KiB of the padded row image lane-linearly, so
+          // lane L of piece p loads whatever belongs at byte p * 1024 + 16 L: row = that / row
+          // bytes, the 16-byte chunk inside the row, or nothing useful in the row's padding
+          // and in rows of masked keys (row 0 of the cache: the score is masked anyway).
+          const int total_b = cg * TK * rowB;
+          int row = drow0, rem = drem0;
+          for (int pb = wave * 1024; pb < total_b; pb += NW * 1024) {
+            const u16* src = a.k;
+            if (row < cg * TK && rem < dq * 2) {
+              const int sl = slot[row & (TK - 1)];
+              src = a.k + (long)(sl >= 0 ? sl : 0) * a.k_stride + (c0 + (row >> 5)) * dq +
+                    (rem >> 1);
             }
-#pragma unroll
-            for (int u = 0; u < STG; ++u)
-              if (lds_off[u] >= 0) *reinterpret_cast<uint4*>(Ks + lds_off[u]) = val[u];
+            __builtin_amdgcn_global_load_lds((gbl_void*)src, (lds_void*)((char*)Ks + pb), 16, 0, 0);
+            row += dq8k;
+            rem += dr8k;
+            if (rem >= rowB) { rem -= rowB; row += 1; }
           }
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         __syncthreads();
 #pragma unroll
@@ -562,7 +560,7 @@ extern "C" int dli_window_attention_mfma(
   if ((size_t)slot_cap * 4 > 16 * 1024) slot_cap = 0;
   const size_t fixed = (wide ? (size_t)NW * TQ * 40
                              : (size_t)TQ * TK * (Hp + 8) + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
-                       (size_t)(slot_cap > TK ? slot_cap : TK) * 4 + 64;
+                       (size_t)(slot_cap > TK ? slot_cap : TK) * 4 + 64 + 1024;
   const size_t per_cg = (size_t)((TK * ldk > dvw * 40) ? TK * ldk : dvw * 40) * 2;
   const size_t budget = 158 * 1024;
   if (fixed + per_cg > budget) return (int)hipErrorNotSupported;

@@ -74,6 +74,8 @@ def buborax_config(c: dict, name: Optional[str] = None) -> ModelConfig:
             raise ValueError(f"unsupported feed-forward kind '{mlp.get('kind')}'")
         ff = int(mlp["ff"]) if mlp else 0
         H, d = int(mx["heads"]), int(mx["dim"])
+        # no mask: every earlier position is visible
+        win = int((mx.get("mask") or {}).get("size") or (1 << 30))
         if kind == "attention":
             G = int(mx.get("kv_heads") or H)
             dv = int(mx.get("vdim", d))
@@ -81,16 +83,15 @@ def buborax_config(c: dict, name: Optional[str] = None) -> ModelConfig:
                 raise ValueError("attention: the values are the keys (vdim == dim) and heads "
                                  "must be a multiple of kv_heads")
             specs.append(LayerSpec("attention", heads=H, kv_heads=G, dim=d, vdim=dv,
-                                   window=int(mx["mask"]["size"]), scale=float(mx["scale"]),
-                                   ff=ff))
+                                   window=win, scale=float(mx.get("scale", d ** -0.5)), ff=ff))
         elif kind == "hgrn2":
             specs.append(LayerSpec("hgrn2", heads=H, dim=d, vdim=int(mx["vdim"]), ff=ff))
         elif kind == "latent_attention":
             rot = mx.get("rot") or {}
             dr = int(mx["rot_dim"])
             specs.append(LayerSpec("latent_attention", heads=H, kv_heads=1, dim=d,
-                                   vdim=int(mx["vdim"]), window=int(mx["mask"]["size"]),
-                                   scale=float(mx["scale"]), rot_dim=dr,
+                                   vdim=int(mx["vdim"]), window=win,
+                                   scale=float(mx.get("scale", (d + dr) ** -0.5)), rot_dim=dr,
                                    kv_rank=int(mx["kv_rank"]), rot_dims=int(rot.get("dims", dr)),
                                    rot_base=float(rot.get("base", 10000.0)), ff=ff))
         else:
