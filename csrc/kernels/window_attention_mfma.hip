@@ -3,7 +3,8 @@
 // 128-wide slice of the value dimension), all heads in the workgroup because the head-mixing
 // matrix needs every head's normalised weights at the same (query, key).
 //
-// Two passes over the window in tiles of 32 keys:
+// With head mixing, two passes over the window in tiles of 32 keys (without it an unsplit
+// launch runs the usual single pass with rescaled accumulators):
 //   pass 1   S^T = K . Q^T per head (v_mfma_f32_16x16x32_bf16, K rows as operand A, so a lane
 //            holds 8 keys of ONE query: max / sum reduce over 2 shuffles), running max m and
 //            sum l per (head, query) in registers.
@@ -159,7 +160,12 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
       l_run[hh] = L;
     }
   }
-  const int pass_lo = a.mode == 2 ? 1 : 0, pass_hi = a.mode == 1 ? 1 : 2;
+  // without head mixing an unsplit launch needs one pass only (see the score phase)
+  // (mode 3: one pass per key split; the split's max / sum go out with its un-normalised
+  // partial output and the reduce kernel weighs the splits)
+  const bool single = wide && (a.mode == 0 || a.mode == 3);
+  const int pass_lo = (a.mode == 2 || single) ? 1 : 0, pass_hi = a.mode == 1 ? 1 : 2;
+  const int rowsT = (int)(a.o_ws_stride / ((long)H * dv));   // rows of a partial-output image
   // staging walks: per-thread start indices and 512-chunk strides, divided once
   const int vcpr = dvc >> 3;
   const int rowB = ldk * 2;                       // bytes of a padded K row in LDS
@@ -295,7 +301,35 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
               sv[kb * 4 + r] = x;
               tmax = fmaxf(tmax, x);
             }
-          if (pass == 0) {
+          if (single) {
+            // one pass (no head mixing, so un-normalised weights can be applied at once):
+            // running max with the accumulators rescaled when it moves, 1 / l at the end
+            tmax = group4_max(tmax);
+            const float m_new = fmaxf(m_run[0], tmax);
+            const float mm = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[0] - mm);
+            float w[8];
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { w[i] = __builtin_amdgcn_exp2f(sv[i] - mm); sum += w[i]; }
+            sum = group4_sum(sum);
+            l_run[0] = l_run[0] * alpha + sum;
+            m_run[0] = m_new;
+            if (alpha != 1.f) {
+#pragma unroll
+              for (int g2 = 0; g2 < MAXHW; ++g2)
+#pragma unroll
+                for (int b = 0; b < MAXDVB; ++b) oacc[g2][b] *= alpha;
+            }
+            u16* dst = Pp + (wave * TQ + fr) * 40 + fq * 4;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+              uint2 pk;
+              pk.x = pack2bf(w[kb * 4], w[kb * 4 + 1]);
+              pk.y = pack2bf(w[kb * 4 + 2], w[kb * 4 + 3]);
+              *reinterpret_cast<uint2*>(dst + kb * 16) = pk;
+            }
+          } else if (pass == 0) {
             tmax = group4_max(tmax);
             const float m_new = fmaxf(m_run[hh], tmax);
             // exp2(-inf - m) = 0 for a finite m; a row with no visible key yet keeps m = -inf
@@ -433,7 +467,12 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
     return;
   }
   if (!my_q) return;
-  if (a.mode == 2) {
+  if (a.mode == 3 && fq == 0 && hbase + wave < H) {
+    float* pr = a.stats_ws + (((long)split * rowsT + t0 + fr) * H + hbase + wave) * 2;
+    pr[0] = m_run[0];
+    pr[1] = l_run[0];
+  }
+  if (a.mode == 2 || a.mode == 3) {
 #pragma unroll
     for (int hh = 0; hh < MAXHW; ++hh) {
       const int h = wide ? hbase + wave : wave + hh * NW;
@@ -449,6 +488,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
     }
     return;
   }
+  const float onorm = single ? (l_run[0] > 0.f ? 1.f / l_run[0] : 0.f) : 1.f;
 #pragma unroll
   for (int hh = 0; hh < MAXHW; ++hh) {
     const int h = wide ? hbase + wave : wave + hh * NW;
@@ -461,7 +501,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
       float o[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        o[r] = oacc[hh][b][r];
+        o[r] = oacc[hh][b][r] * onorm;
         if (a.gate != nullptr)
           o[r] *= 1.f / (1.f + expf(-a.gate[(long)(t0 + fr) * a.ldg + col + r]));
       }
@@ -476,14 +516,30 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
 // out[t][c] = bf16(gate * sum over splits of the partial outputs), 4 columns a thread
 __global__ void __launch_bounds__(256) split_reduce_kernel(
     u16* __restrict__ out, int ldo, const float* __restrict__ o_ws, long stride, int nsplit,
-    const float* __restrict__ gate, int ldg, int T, int width) {
+    const float* __restrict__ gate, int ldg, int T, int width, const float* __restrict__ stats,
+    int H, int dv) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int w4 = width >> 2;
   if (gid >= (long)T * w4) return;
   const int t = (int)(gid / w4), c = (int)(gid % w4) * 4;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int k = 0; k < nsplit; ++k)
-    acc += *reinterpret_cast<const f32x4*>(o_ws + k * stride + (long)t * width + c);
+  if (stats != nullptr) {
+    // un-normalised partials with their own (max, sum) in the log2 domain
+    const int h = c / dv;
+    float M = -INFINITY, L = 0.f;
+    for (int k = 0; k < nsplit; ++k) M = fmaxf(M, stats[(((long)k * T + t) * H + h) * 2]);
+    for (int k = 0; k < nsplit; ++k) {
+      const float* pr = stats + (((long)k * T + t) * H + h) * 2;
+      if (pr[0] == -INFINITY) continue;
+      const float wk = __builtin_amdgcn_exp2f(pr[0] - M);
+      L += pr[1] * wk;
+      acc += wk * *reinterpret_cast<const f32x4*>(o_ws + k * stride + (long)t * width + c);
+    }
+    acc *= L > 0.f ? 1.f / L : 0.f;
+  } else {
+    for (int k = 0; k < nsplit; ++k)
+      acc += *reinterpret_cast<const f32x4*>(o_ws + k * stride + (long)t * width + c);
+  }
   if (gate != nullptr) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[r] *= 1.f / (1.f + expf(-gate[(long)t * ldg + c + r]));
@@ -521,7 +577,9 @@ extern "C" long dli_window_attention_mfma_workspace_bytes(int num_seqs, int max_
   const int nsplit = pick_splits(num_seqs, max_seqlen, H, dv, window, mixing == 0);
   if (nsplit == 1) return 0;
   const long qtiles = (max_seqlen + TQ - 1) / TQ;
-  return ((long)num_seqs * qtiles * nsplit * H * TQ * 2 + (long)nsplit * T * H * dv) * 4;
+  const long st_tiles = (long)num_seqs * qtiles * nsplit * H * TQ * 2;   // two-pass form
+  const long st_rows = (long)nsplit * T * H * 2;                          // one-pass form
+  return ((st_tiles > st_rows ? st_tiles : st_rows) + (long)nsplit * T * H * dv) * 4;
 }
 
 // Returns hipErrorNotSupported (801) when the shapes do not fit this form; the caller then
@@ -598,16 +656,27 @@ extern "C" int dli_window_attention_mfma(
   if (T <= 0 || (H * dv) % 4 || ldo % 4) return (int)hipErrorInvalidValue;
   a.nsplit = nsplit;
   a.stats_ws = (float*)ws;
-  a.o_ws = a.stats_ws + (long)num_seqs * qtiles * nsplit * H * TQ * 2;
+  {
+    const long st_tiles = (long)num_seqs * qtiles * nsplit * H * TQ * 2;
+    const long st_rows = (long)nsplit * T * H * 2;
+    a.o_ws = a.stats_ws + (st_tiles > st_rows ? st_tiles : st_rows);
+  }
   a.o_ws_stride = (long)T * H * dv;
+  const long quads = (long)T * (H * dv / 4);
+  if (wide) {            // no mixing: one pass per split, the reduce weighs the splits
+    a.mode = 3;
+    WA_LAUNCH(dim3(qtiles, num_seqs, ndvs * nhs * nsplit));
+    split_reduce_kernel<<<(int)((quads + 255) / 256), 256, 0, st>>>(
+        (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv, a.stats_ws, H, dv);
+    DLI_RETURN_LAUNCH();
+  }
   a.mode = 1;
   a.ndvs = 1;                                     // the statistics do not depend on the slice
   WA_LAUNCH(dim3(qtiles, num_seqs, nhs * nsplit));
   a.mode = 2;
   a.ndvs = ndvs;
   WA_LAUNCH(dim3(qtiles, num_seqs, ndvs * nhs * nsplit));
-  const long quads = (long)T * (H * dv / 4);
   split_reduce_kernel<<<(int)((quads + 255) / 256), 256, 0, st>>>(
-      (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv);
+      (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv, nullptr, H, dv);
   DLI_RETURN_LAUNCH();
 }
