@@ -13,10 +13,14 @@
 //            lands as Pp[head][query][key]; then O += W' . V with W' rows as operand A and the
 //            V tile, staged transposed (Vt[dim][key]), as operand B.
 // With mixing, heads are dealt to waves round-robin (head h -> wave h % 8, at most 4 heads a
-// wave, H <= 32, 128-wide value slices); without it, the wide form takes 8 heads a workgroup;
-// the key / value tiles are staged per group of kv heads that fits the LDS budget. Query
-// fragments are re-read from global memory (L2) per use: with 576-wide latent queries they do
-// not fit registers, and the LDS is taken by the weight tiles.
+// wave, H <= 32, 128-wide value slices); without it, the wide form takes 8 heads a workgroup.
+// Staging: the cache rows of the whole window are looked up once (slot table in LDS); a tile's
+// K rows of every kv head that fits go to LDS by LDS-DMA (global_load_lds_dwordx4, padded rows,
+// all pieces in flight); the V tile shares that LDS region (the two are never live together)
+// and is transposed through registers. Query fragments come from global memory (L2), four at
+// a time, the first group of a step requested together with the K tile: with 576-wide latent
+// queries they fit neither registers nor the LDS left beside the weight tiles.
+// Scores live in the log2 domain (scale and slope carry log2 e): one v_exp_f32 per weight.
 //
 // Masked positions (outside the window, after the query, past the sequence, rows past the
 // tile's last query) get weight 0; a query row always sees itself, so l > 0.
