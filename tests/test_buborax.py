@@ -446,3 +446,18 @@ def test_generation_under_preemption(device, dtype):
             seq.append(tok)
         assert len(o.output_ids) == new
     assert eng.bm.num_free == eng.bm.num_blocks and eng.state_slots.num_free == 3
+
+
+def test_registry_model_random_init_generates():
+    """The registry's test-size hybrid (``buborax-tiny``) through the plain entry point: random
+    init by name, prompts as text (byte tokenizer), sampled generation, deterministic per seed."""
+    outs = []
+    for _ in range(2):
+        eng = LLMEngine("buborax-tiny", device="cpu", dtype=torch.float32, max_batch=4,
+                        max_model_len=64, block_size=8, num_blocks=64, seed=3)
+        o = eng.generate(["hybrid", "layers"], SamplingParams(max_new_tokens=6, seed=11,
+                                                              ignore_eos=True))
+        assert all(len(x.output_ids) == 6 for x in o)
+        assert all(0 <= t < eng.cfg.vocab_size for x in o for t in x.output_ids)
+        outs.append([x.output_ids for x in o])
+    assert outs[0] == outs[1]
