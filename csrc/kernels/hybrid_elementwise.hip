@@ -6,10 +6,17 @@
 // that storage type; residuals, projection outputs that feed a norm, a gate or a recurrence,
 // and all arithmetic are fp32 in both.
 //
-//  * embedding_f32      x[t] = table[ids[t]] as fp32 (two copies: the stream and the loop input)
-//  * resadd_groupnorm   x = keep * x + mult * y + bias; h = grouped RMS norm of x (S out)
+//  * embedding_f32      x[t] = table[ids[t]] * scale (+ pos_table[positions[t]]) as fp32 (two
+//                       copies: the stream and the loop input)
+//  * resadd_groupnorm   x = keep * x + mult * y + bias; h = grouped RMS norm of x * gain (S out,
+//                       or unrounded fp32 for a consumer that mixes rows first)
+//  * token_shift        u[t] = h[t] + (h[t-1] - h[t]) * mu over the normed fp32 rows, h[t-1] of a
+//                       portion's first row from the sequence's state slot
+//  * talk_prepare       q / k / v bias, unit-RMS q and k heads, k and v -> cache, queries with
+//                       the pre-softmax head mixing folded in -> S
 //  * concat_cast        [x ; x0] fp32 -> S rows of width 2D (the operand of the loop-entry GEMM)
-//  * gelu_mul           gelu_tanh(gate) * up over a [T, 2F] fp32 projection -> S [T, F]
+//  * act_mul            gelu_tanh(gate) * up, silu(gate) * up or gelu_tanh(up) over a fp32
+//                       projection -> S [T, F]
 //  * attn_prepare       per-head RMS norm of q and k (shared weights), normed k -> key cache,
 //                       raw k -> value cache ("values are the keys"), normed q -> S
 //  * mla_prepare        latent attention: RMS norm of the compressed kv -> cache, interleaved
@@ -29,13 +36,19 @@ template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p =
 template <typename S>
 __global__ void __launch_bounds__(256) embedding_f32_kernel(
     float* __restrict__ x, float* __restrict__ x0, const int* __restrict__ ids,
-    const S* __restrict__ table, int T, int dim, int vocab) {
+    const S* __restrict__ table, int T, int dim, int vocab, float scale,
+    const S* __restrict__ pos_table, const int* __restrict__ positions, int max_pos) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= (long)T * dim) return;
   const int t = (int)(gid / dim), c = (int)(gid % dim);
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-  const float v = ldf(table + (long)id * dim + c);
+  float v = ldf(table + (long)id * dim + c) * scale;
+  if (pos_table != nullptr) {
+    int p = positions[t];
+    p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+    v += ldf(pos_table + (long)p * dim + c);
+  }
   x[gid] = v;
   if (x0 != nullptr) x0[gid] = v;
 }
@@ -47,8 +60,9 @@ __global__ void __launch_bounds__(256) embedding_f32_kernel(
 template <typename S>
 __global__ void __launch_bounds__(256) resadd_groupnorm_kernel(
     float* __restrict__ x, const float* __restrict__ y, int ldy, const S* __restrict__ bias,
-    float keep, float mult, const S* __restrict__ w, S* __restrict__ h, int ldh, int dim,
-    int groups, float eps, const long* __restrict__ rows_idx, bool vec4) {
+    float keep, float mult, const S* __restrict__ w, void* __restrict__ h, int ldh, int dim,
+    int groups, float eps, const long* __restrict__ rows_idx, bool vec4, float gain,
+    bool h_f32) {
   extern __shared__ __attribute__((aligned(16))) float row[];   // dim floats + group scales
   float* gsum = row + dim;
   const int r = blockIdx.x;
@@ -95,8 +109,47 @@ __global__ void __launch_bounds__(256) resadd_groupnorm_kernel(
     if (lane == 0) gsum[g] = 1.f / sqrtf(s / (float)gl + eps);
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < dim; c += blockDim.x)
-    stf(h + (long)r * ldh + c, row[c] * gsum[c / gl] * ldf(w + c));
+  if (h_f32) {
+    for (int c = threadIdx.x; c < dim; c += blockDim.x)
+      ((float*)h)[(long)r * ldh + c] = row[c] * gsum[c / gl] * ldf(w + c) * gain;
+  } else {
+    for (int c = threadIdx.x; c < dim; c += blockDim.x)
+      stf((S*)h + (long)r * ldh + c, row[c] * gsum[c / gl] * ldf(w + c) * gain);
+  }
+}
+
+// Token shift over normed fp32 rows: u[t] = h[t] + (h[t-1] - h[t]) * mu. Grid (row blocks of a
+// sequence, sequences). h[t-1] of a portion's first row is the sequence's row of `state`
+// (zeros at position 0). The workgroup that holds a portion's first row also stores the
+// portion's LAST row into the state, after it has read the old one: every thread reads and
+// then writes the same columns, so the order holds without a second launch. Sequences
+// without a slot (padding rows of a captured step) pass through unshifted.
+constexpr int SHIFT_ROWS = 4;
+template <typename S>
+__global__ void __launch_bounds__(256) token_shift_kernel(
+    const float* __restrict__ h, const S* __restrict__ mu, float* __restrict__ state,
+    const int* __restrict__ slots, const int* __restrict__ cu, const int* __restrict__ positions,
+    S* __restrict__ out, int dim) {
+  const int s = blockIdx.y;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  const int r0 = blockIdx.x * SHIFT_ROWS;
+  if (t0 + r0 >= t1) return;
+  const int slot = slots != nullptr ? slots[s] : -1;
+  const int rows = min(SHIFT_ROWS, t1 - t0 - r0);
+  const bool from_zero = positions[t0] == 0;
+  for (int c = threadIdx.x; c < dim; c += blockDim.x) {
+    const float m = ldf(mu + c);
+    float prev;
+    if (r0 > 0) prev = h[(long)(t0 + r0 - 1) * dim + c];
+    else prev = (slot < 0 || from_zero) ? 0.f : state[(long)slot * dim + c];
+    for (int i = 0; i < rows; ++i) {
+      const long o = (long)(t0 + r0 + i) * dim + c;
+      const float cur = h[o];
+      stf(out + o, slot < 0 ? cur : cur + (prev - cur) * m);
+      prev = cur;
+    }
+    if (r0 == 0 && slot >= 0) state[(long)slot * dim + c] = h[(long)(t1 - 1) * dim + c];
+  }
 }
 
 template <typename S>
@@ -113,29 +166,92 @@ __device__ __forceinline__ float gelu_tanh32(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
+__device__ __forceinline__ float act_pair(int kind, float g, float u) {
+  if (kind == 0) return gelu_tanh32(g) * u;
+  if (kind == 1) return g / (1.f + expf(-g)) * u;
+  return gelu_tanh32(g);
+}
+
+// kind 0: gelu_tanh(gu[:, c]) * gu[:, F + c]; 1: silu(..) * ..; 2: gelu_tanh(gu[:, c]).
+// nrows (nullable, device): rows from *nrows on hold no data and are skipped.
 template <typename S>
-__global__ void __launch_bounds__(256) gelu_mul_kernel(
-    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F) {
+__global__ void __launch_bounds__(256) act_mul_kernel(
+    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F, int kind,
+    const int* __restrict__ nrows) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= (long)T * F) return;
   const int t = (int)(gid / F), c = (int)(gid % F);
+  if (nrows != nullptr && t >= *nrows) return;
   const float* r = gu + (long)t * ldg;
-  stf(out + (long)t * ldo + c, gelu_tanh32(r[c]) * r[F + c]);
+  stf(out + (long)t * ldo + c, act_pair(kind, r[c], kind == 2 ? 0.f : r[F + c]));
 }
 
 // 4 features a thread (F, ldg multiples of 4, 16-byte aligned rows): 16-byte loads
 template <typename S>
-__global__ void __launch_bounds__(256) gelu_mul4_kernel(
-    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F) {
+__global__ void __launch_bounds__(256) act_mul4_kernel(
+    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F, int kind,
+    const int* __restrict__ nrows) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int f4 = F >> 2;
   if (gid >= (long)T * f4) return;
   const int t = (int)(gid / f4), c = (int)(gid % f4) * 4;
+  if (nrows != nullptr && t >= *nrows) return;
   const float* r = gu + (long)t * ldg;
   const f32x4 g = *reinterpret_cast<const f32x4*>(r + c);
-  const f32x4 u = *reinterpret_cast<const f32x4*>(r + F + c);
+  f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (kind != 2) u = *reinterpret_cast<const f32x4*>(r + F + c);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) stf(out + (long)t * ldo + c + i, gelu_tanh32(g[i]) * u[i]);
+  for (int i = 0; i < 4; ++i) stf(out + (long)t * ldo + c + i, act_pair(kind, g[i], u[i]));
+}
+
+// One workgroup per token. proj row (fp32, + bias): [H*d q | G*d k | G*dv v] (q only when the
+// layer attends another layer's cache: kcache null). q and k heads are divided by their RMS;
+// k and v go to the cache row; the queries leave with the pre-softmax head mixing folded in:
+//   sum_g talk[h][g] (q_g . k_c(g)) = sum_c (sum_{g in c} talk[h][g] q_g) . k_c
+// so head h carries q'_h [G*d] whose part c is sum_{g in c} talk[h][g] q_g, and scores whole
+// cached key rows.
+template <typename S>
+__global__ void __launch_bounds__(256) talk_prepare_kernel(
+    const float* __restrict__ proj, int ldp, const S* __restrict__ bias,
+    const float* __restrict__ talk, float eps, int H, int G, int d, int dv,
+    S* __restrict__ q_out, S* __restrict__ kcache, S* __restrict__ vcache,
+    const int* __restrict__ slots) {
+  extern __shared__ float qn[];                       // [H * d] unit-RMS queries
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const float* row = proj + (long)t * ldp;
+  const int slot = kcache != nullptr ? slots[t] : -1;
+  const int units = H + (slot >= 0 ? G : 0);
+  for (int u = wid; u < units; u += nw) {
+    const int off = u * d;                            // q heads, then k heads, are contiguous
+    float ss = 0.f;
+    for (int c = lane; c < d; c += 64) { const float v = row[off + c] + ldf(bias + off + c); ss += v * v; }
+    ss = wave_sum(ss);
+    const float rs = 1.f / sqrtf(ss / (float)d + eps);
+    if (u < H) {
+      for (int c = lane; c < d; c += 64) qn[off + c] = (row[off + c] + ldf(bias + off + c)) * rs;
+    } else {
+      S* kd = kcache + ((long)slot * G + (u - H)) * d;
+      for (int c = lane; c < d; c += 64) stf(kd + c, (row[off + c] + ldf(bias + off + c)) * rs);
+    }
+  }
+  if (slot >= 0) {
+    const int voff = (H + G) * d;
+    S* vd = vcache + (long)slot * G * dv;
+    for (int c = threadIdx.x; c < G * dv; c += blockDim.x)
+      stf(vd + c, row[voff + c] + ldf(bias + voff + c));
+  }
+  __syncthreads();
+  const int rep = H / G, wq = G * d;
+  S* qo = q_out + (long)t * H * wq;
+  for (int i = threadIdx.x; i < H * wq; i += blockDim.x) {
+    const int h = i / wq, rem = i % wq, c = rem / d, col = rem % d;
+    const float* tk = talk + h * H + c * rep;
+    const float* qs = qn + (c * rep) * d + col;
+    float acc = 0.f;
+    for (int r = 0; r < rep; ++r) acc += tk[r] * qs[r * d];
+    stf(qo + i, acc);
+  }
 }
 
 // proj row: [H*d q | G*d k | ...]; one wave per (token, head) unit, H + G units per token.
@@ -234,19 +350,28 @@ __global__ void __launch_bounds__(256) mla_prepare_kernel(
   } while (0)
 
 extern "C" int dli_embedding_f32(float* x, float* x0, const int* ids, const void* table, int T,
-                                 int dim, int vocab, int dt, hipStream_t st) {
+                                 int dim, int vocab, float scale, const void* pos_table,
+                                 const int* positions, int max_pos, int dt, hipStream_t st) {
   if (T <= 0) return 0;
+  if (pos_table != nullptr && (positions == nullptr || max_pos < 1))
+    return (int)hipErrorInvalidValue;
   const int nb = (int)(((long)T * dim + 255) / 256);
   DT_SWITCH(dt,
-            (embedding_f32_kernel<u16><<<nb, 256, 0, st>>>(x, x0, ids, (const u16*)table, T, dim, vocab)),
-            (embedding_f32_kernel<float><<<nb, 256, 0, st>>>(x, x0, ids, (const float*)table, T, dim, vocab)));
+            (embedding_f32_kernel<u16><<<nb, 256, 0, st>>>(x, x0, ids, (const u16*)table, T, dim,
+                                                          vocab, scale, (const u16*)pos_table,
+                                                          positions, max_pos)),
+            (embedding_f32_kernel<float><<<nb, 256, 0, st>>>(x, x0, ids, (const float*)table, T,
+                                                            dim, vocab, scale,
+                                                            (const float*)pos_table, positions,
+                                                            max_pos)));
   DLI_RETURN_LAUNCH();
 }
 
 extern "C" int dli_resadd_groupnorm(float* x, const float* y, int ldy, const void* bias,
                                     float keep, float mult, const void* w, void* h, int ldh,
                                     int rows, int dim, int groups, float eps,
-                                    const long* rows_idx, int dt, hipStream_t st) {
+                                    const long* rows_idx, float gain, int h_f32, int dt,
+                                    hipStream_t st) {
   if (rows <= 0) return 0;
   if (groups < 1 || dim % groups || (size_t)(dim + groups) * 4 > 60000)
     return (int)hipErrorInvalidValue;
@@ -255,11 +380,11 @@ extern "C" int dli_resadd_groupnorm(float* x, const float* y, int ldy, const voi
                     (y == nullptr || ((uintptr_t)y % 16 == 0 && ldy % 4 == 0));
   DT_SWITCH(dt,
             (resadd_groupnorm_kernel<u16><<<rows, 256, sh, st>>>(
-                x, y, ldy, (const u16*)bias, keep, mult, (const u16*)w, (u16*)h, ldh, dim, groups,
-                eps, rows_idx, vec4)),
+                x, y, ldy, (const u16*)bias, keep, mult, (const u16*)w, h, ldh, dim, groups,
+                eps, rows_idx, vec4, gain, h_f32 != 0)),
             (resadd_groupnorm_kernel<float><<<rows, 256, sh, st>>>(
-                x, y, ldy, (const float*)bias, keep, mult, (const float*)w, (float*)h, ldh, dim,
-                groups, eps, rows_idx, vec4)));
+                x, y, ldy, (const float*)bias, keep, mult, (const float*)w, h, ldh, dim,
+                groups, eps, rows_idx, vec4, gain, h_f32 != 0)));
   DLI_RETURN_LAUNCH();
 }
 
@@ -272,18 +397,53 @@ extern "C" int dli_concat_cast(void* out, const float* a, const float* b, int T,
   DLI_RETURN_LAUNCH();
 }
 
-extern "C" int dli_gelu_mul(void* out, int ldo, const float* gu, int ldg, int T, int F, int dt,
-                            hipStream_t st) {
+extern "C" int dli_token_shift(const float* h, const void* mu, float* state, const int* slots,
+                               const int* cu, const int* positions, void* out, int num_seqs,
+                               int max_seqlen, int dim, int dt, hipStream_t st) {
+  if (num_seqs <= 0 || max_seqlen <= 0) return 0;
+  if (num_seqs > 65535) return (int)hipErrorInvalidValue;
+  dim3 grid((max_seqlen + SHIFT_ROWS - 1) / SHIFT_ROWS, num_seqs);
+  DT_SWITCH(dt,
+            (token_shift_kernel<u16><<<grid, 256, 0, st>>>(h, (const u16*)mu, state, slots, cu,
+                                                          positions, (u16*)out, dim)),
+            (token_shift_kernel<float><<<grid, 256, 0, st>>>(h, (const float*)mu, state, slots, cu,
+                                                            positions, (float*)out, dim)));
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_act_mul(void* out, int ldo, const float* gu, int ldg, int T, int F, int kind,
+                           const int* nrows, int dt, hipStream_t st) {
   if (T <= 0) return 0;
+  if (kind < 0 || kind > 2) return (int)hipErrorInvalidValue;
   if (F % 4 == 0 && ldg % 4 == 0 && (uintptr_t)gu % 16 == 0) {
     const int nb4 = (int)(((long)T * (F / 4) + 255) / 256);
-    DT_SWITCH(dt, (gelu_mul4_kernel<u16><<<nb4, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F)),
-              (gelu_mul4_kernel<float><<<nb4, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F)));
+    DT_SWITCH(dt,
+              (act_mul4_kernel<u16><<<nb4, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows)),
+              (act_mul4_kernel<float><<<nb4, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows)));
     DLI_RETURN_LAUNCH();
   }
   const int nb = (int)(((long)T * F + 255) / 256);
-  DT_SWITCH(dt, (gelu_mul_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F)),
-            (gelu_mul_kernel<float><<<nb, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F)));
+  DT_SWITCH(dt, (act_mul_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows)),
+            (act_mul_kernel<float><<<nb, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows)));
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_talk_prepare(const float* proj, int ldp, const void* bias, const float* talk,
+                                float eps, int T, int H, int G, int d, int dv, void* q_out,
+                                void* kcache, void* vcache, const int* slots, int dt,
+                                hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H < 1 || G < 1 || H % G || d < 1 || dv < 1 || (kcache == nullptr) != (vcache == nullptr))
+    return (int)hipErrorInvalidValue;
+  const size_t sh = (size_t)H * d * 4;
+  if (sh > 60000) return (int)hipErrorInvalidValue;
+  DT_SWITCH(dt,
+            (talk_prepare_kernel<u16><<<T, 256, sh, st>>>(
+                proj, ldp, (const u16*)bias, talk, eps, H, G, d, dv, (u16*)q_out, (u16*)kcache,
+                (u16*)vcache, slots)),
+            (talk_prepare_kernel<float><<<T, 256, sh, st>>>(
+                proj, ldp, (const float*)bias, talk, eps, H, G, d, dv, (float*)q_out,
+                (float*)kcache, (float*)vcache, slots)));
   DLI_RETURN_LAUNCH();
 }
 

@@ -405,3 +405,125 @@ extern "C" int dli_ep_pack(void* send_x, int* send_e, int* pos, int* fill, const
                                          ids, k, D, e_per);
   DLI_RETURN_LAUNCH();
 }
+
+
+// ---------------------------------------------------------------------------------------------
+// Router of a mixture whose weights are the un-renormalised softmax scores and whose choice
+// adds a learned correction (score_router), for any storage type (dt 0 bf16, 1 fp32):
+//   z = W[:n] h (fp32), s = softmax(z) over all n experts, the `top` largest of s + corr are
+//   chosen (lowest index on ties), weights = s of the chosen. Rows n .. n + n_gate - 1 of W are
+//   extra per-token gates: sigmoid(W[r] h).
+// One workgroup per token: the row sits in LDS as fp32, each wave takes router rows in turn
+// (lanes stride the row, one shuffle reduce: a fixed order, whatever else is in the batch),
+// thread 0 then runs the softmax and the `top` selection rounds over the n <= 1024 scores.
+// A row of NaNs still selects valid ids (0 .. top-1), so a padding row cannot send the
+// expert GEMMs out of range.
+namespace {
+
+template <typename S> __device__ __forceinline__ float rld(const S* p);
+template <> __device__ __forceinline__ float rld<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float rld<float>(const float* p) { return *p; }
+
+constexpr int ROUTER_MAX = 1024;
+
+template <typename S>
+__global__ void __launch_bounds__(256) score_router_kernel(
+    float* __restrict__ topk_w, int* __restrict__ topk_ids, float* __restrict__ gates,
+    const S* __restrict__ h, int ldh, const S* __restrict__ W, const float* __restrict__ corr,
+    int D, int n, int n_gate, int top) {
+  extern __shared__ float rsm[];                      // [D] row, [n + n_gate] logits
+  float* row = rsm;
+  float* z = rsm + D;
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) row[c] = rld(h + (long)t * ldh + c);
+  __syncthreads();
+  for (int e = wid; e < n + n_gate; e += nw) {
+    const S* wr = W + (long)e * D;
+    float acc = 0.f;
+    for (int c = lane; c < D; c += 64) acc += row[c] * rld(wr + c);
+    acc = wave_sum(acc);
+    if (lane == 0) z[e] = acc;
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  float m = -INFINITY;
+  for (int e = 0; e < n; ++e) m = fmaxf(m, z[e]);
+  float sum = 0.f;
+  for (int e = 0; e < n; ++e) { const float v = expf(z[e] - m); z[e] = v; sum += v; }
+  const float inv = 1.f / sum;
+  for (int g = 0; g < n_gate; ++g) gates[(long)t * n_gate + g] = 1.f / (1.f + expf(-z[n + g]));
+  // selection rounds; a chosen expert's score is kept aside and its slot marked with -2
+  for (int j = 0; j < top; ++j) {
+    int best = -1;
+    float bc = -INFINITY;
+    for (int e = 0; e < n; ++e) {
+      const float sc = z[e];
+      if (sc == -2.f) continue;
+      const float c = sc * inv + corr[e];
+      if (best < 0 || c > bc) { best = e; bc = c; }
+    }
+    topk_ids[(long)t * top + j] = best;
+    topk_w[(long)t * top + j] = z[best] * inv;
+    z[best] = -2.f;
+  }
+}
+
+// out[t] = sum_j w[t][j] * (routed ? y[pos[t][j]] : identity ? x[t] : 0) + gate[t] * ys[t]
+// y, ys fp32; x storage type; ids >= n_real are identity experts (their pos is -1).
+template <typename S>
+__global__ void __launch_bounds__(256) moe_combine_f32_kernel(
+    float* __restrict__ out, const float* __restrict__ y, const float* __restrict__ w,
+    const int* __restrict__ pos, const int* __restrict__ ids, const S* __restrict__ x, int ldx,
+    const float* __restrict__ ys, const float* __restrict__ gate, int ldg, int T, int k, int dim,
+    int n_real) {
+  const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (long)T * dim) return;
+  const int t = (int)(gid / dim), c = (int)(gid % dim);
+  float acc = 0.f;
+  for (int j = 0; j < k; ++j) {
+    const int p = pos[t * k + j];
+    const float ww = w[t * k + j];
+    if (p >= 0) acc += ww * y[(long)p * dim + c];
+    else if (ids[t * k + j] >= n_real) acc += ww * rld(x + (long)t * ldx + c);
+  }
+  if (ys != nullptr) acc += gate[(long)t * ldg] * ys[(long)t * dim + c];
+  out[gid] = acc;
+}
+
+}  // namespace
+
+extern "C" int dli_score_router(float* topk_w, int* topk_ids, float* gates, const void* h, int ldh,
+                                const void* W, const float* corr, int T, int D, int n, int n_gate,
+                                int top, int dt, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (n < 1 || n_gate < 0 || top < 1 || top > n || n + n_gate > ROUTER_MAX ||
+      (size_t)(D + n + n_gate) * 4 > 60000)
+    return (int)hipErrorInvalidValue;
+  const size_t sh = (size_t)(D + n + n_gate) * 4;
+  if (dt == 0)
+    score_router_kernel<u16><<<T, 256, sh, st>>>(topk_w, topk_ids, gates, (const u16*)h, ldh,
+                                                 (const u16*)W, corr, D, n, n_gate, top);
+  else if (dt == 1)
+    score_router_kernel<float><<<T, 256, sh, st>>>(topk_w, topk_ids, gates, (const float*)h, ldh,
+                                                   (const float*)W, corr, D, n, n_gate, top);
+  else return (int)hipErrorInvalidValue;
+  DLI_RETURN_LAUNCH();
+}
+
+extern "C" int dli_moe_combine_f32(float* out, const float* y, const float* w, const int* pos,
+                                   const int* ids, const void* x, int ldx, const float* ys,
+                                   const float* gate, int ldg, int T, int k, int dim, int n_real,
+                                   int dt, hipStream_t st) {
+  if (T <= 0) return 0;
+  if ((ys == nullptr) != (gate == nullptr)) return (int)hipErrorInvalidValue;
+  const int nb = (int)(((long)T * dim + 255) / 256);
+  if (dt == 0)
+    moe_combine_f32_kernel<u16><<<nb, 256, 0, st>>>(out, y, w, pos, ids, (const u16*)x, ldx, ys,
+                                                    gate, ldg, T, k, dim, n_real);
+  else if (dt == 1)
+    moe_combine_f32_kernel<float><<<nb, 256, 0, st>>>(out, y, w, pos, ids, (const float*)x, ldx,
+                                                      ys, gate, ldg, T, k, dim, n_real);
+  else return (int)hipErrorInvalidValue;
+  DLI_RETURN_LAUNCH();
+}

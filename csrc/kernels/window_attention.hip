@@ -11,6 +11,11 @@
 //                     kernel makes two passes over the window: (1) running max / sum per head,
 //                     (2) weights, mix, weighted value sum.
 //  * gate    != null: out *= sigmoid(gate) (fp32 pre-activation of the same token, ldg)
+//  * chunk   > 0: a query also sees only the keys of its own block of `chunk` positions
+//                     (blocks counted from position 0 of the sequence)
+//  * Gk != G: the key rows hold Gk heads of dq while the values hold G heads of dv (Gk = 1:
+//                     every query head scores the whole key row — head mixing before the
+//                     softmax folded into the queries)
 //  * dq != dv, and v_cache may alias k_cache with its own row stride: latent attention in the
 //    absorbed form reads one [latent | rotated key] row per token, scores over all of it and
 //    values = its first dv columns (G = 1: every head shares the row).
@@ -47,6 +52,7 @@ struct WinAttnArgs {
   const int* block_tables; int bt_stride; int block_size;
   int H, G, dq, dv, window;
   float scale;
+  int Gk, chunk;
 };
 
 template <typename S>
@@ -63,14 +69,15 @@ __global__ void __launch_bounds__(256) window_attention_kernel(WinAttnArgs a) {
   const int t = a.cu[s] + blockIdx.x;
   if (t >= a.cu[s + 1]) return;
   const int p = a.positions[t];
-  const int lo = max(0, p - a.window + 1);
+  int lo = max(0, p - a.window + 1);
+  if (a.chunk > 0) lo = max(lo, p / a.chunk * a.chunk);
   const int n = p + 1 - lo;
   const int tid = threadIdx.x;
   const S* qrow = (const S*)a.q + (long)t * a.ldq;
   for (int i = tid; i < H * dq; i += blockDim.x) qs[i] = ldf(qrow + i);
   for (int h = tid; h < H; h += blockDim.x) { hm[h] = -INFINITY; hl[h] = 0.f; }
   const int* bt = a.block_tables + (long)s * a.bt_stride;
-  const int hpg = H / G;
+  const int hpg = H / G, hpk = H / a.Gk;
   float acc[MAX_ACC];
 #pragma unroll
   for (int i = 0; i < MAX_ACC; ++i) acc[i] = 0.f;
@@ -90,7 +97,7 @@ __global__ void __launch_bounds__(256) window_attention_kernel(WinAttnArgs a) {
         const int sl = slot[jj];
         float sc = -INFINITY;
         if (sl >= 0) {
-          const S* kr = (const S*)a.k + (long)sl * a.k_stride + (h / hpg) * dq;
+          const S* kr = (const S*)a.k + (long)sl * a.k_stride + (h / hpk) * dq;
           const float* qh = qs + h * dq;
           float d0 = 0.f;
           for (int c = 0; c < dq; ++c) d0 += qh[c] * ldf(kr + c);
@@ -166,10 +173,11 @@ extern "C" int dli_window_attention(
     const void* q, int ldq, const void* k, long k_stride, const void* v, long v_stride, void* out,
     int ldo, const float* gate, int ldg, const float* slopes, const float* talk, const int* cu,
     const int* positions, const int* block_tables, int bt_stride, int block_size, int num_seqs,
-    int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int dt,
-    hipStream_t st) {
+    int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int Gk, int chunk,
+    int dt, hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
-  if (H < 1 || G < 1 || H % G || dq < 1 || dv < 1 || window < 1 || block_size < 1 ||
+  if (H < 1 || G < 1 || H % G || Gk < 1 || H % Gk || chunk < 0 || dq < 1 || dv < 1 ||
+      window < 1 || block_size < 1 ||
       (long)H * dv > 256L * MAX_ACC)
     return (int)hipErrorInvalidValue;
   const size_t sh = ((size_t)H * dq + 2 * (size_t)H * KT + 2 * H + KT) * 4;
@@ -186,7 +194,8 @@ extern "C" int dli_window_attention(
     }
   }
   WinAttnArgs a{q, ldq, k, k_stride, v, v_stride, out, ldo, gate, ldg, slopes, talk, cu,
-                positions, block_tables, bt_stride, block_size, H, G, dq, dv, window, scale};
+                positions, block_tables, bt_stride, block_size, H, G, dq, dv, window, scale,
+                Gk, chunk};
   dim3 grid(max_seqlen, num_seqs);
   if (dt == 0) window_attention_kernel<u16><<<grid, 256, sh, st>>>(a);
   else if (dt == 1) window_attention_kernel<float><<<grid, 256, sh, st>>>(a);

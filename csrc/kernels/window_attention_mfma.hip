@@ -593,8 +593,10 @@ extern "C" int dli_window_attention_mfma(
     int ldo, const float* gate, int ldg, const float* slopes, const float* talk, const int* cu,
     const int* positions, const int* block_tables, int bt_stride, int block_size, int num_seqs,
     int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int T, void* ws,
-    int rowhead, hipStream_t st) {
+    int rowhead, int Gk, int chunk, hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
+  // block masks and key rows whose head count differs from the values' run the scalar form
+  if (chunk != 0 || Gk != G) return (int)hipErrorNotSupported;
   int rowmul = 1;
   if (rowhead) {
     if (talk != nullptr || gate != nullptr || slopes != nullptr || G != 1 || max_seqlen != 1 ||

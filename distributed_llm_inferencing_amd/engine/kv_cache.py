@@ -93,6 +93,12 @@ class HybridCache:
                             block * block_size + offset; k holds the normed keys, v the raw ones
     * ``latent_attention``: (c [slots, kv_rank + rot_dim],)     normed latent | rotated key
     * ``hgrn2``:            (state [state_slots, H, d, dv] fp32,)  one slot per live sequence
+    * ``talk_attention``:   (k [slots, G*d], v [slots, G*dv])   normed keys and values; a layer
+                            with ``kv_from`` gets the tensors of that layer's run (it writes
+                            nothing)
+
+    ``shift_states[run]`` is [state_slots, D] fp32 for a layer with token shift (the previous
+    token's mixer input), else None.
 
     Rows are zero-initialised once (padding rows of captured decode steps read row 0). A state
     slot is not cleared on reuse: a sequence's first portion starts from zero by position."""
@@ -106,8 +112,23 @@ class HybridCache:
         self.num_layers = len(cfg.layer_runs())
         rows = num_blocks * block_size
         self.entries = []
-        for li, _, _ in cfg.layer_runs():
+        self.shift_states = []
+        run_of = {}                       # layer -> its (last) run, for layers that lend their cache
+        for ri, (li, _, _) in enumerate(cfg.layer_runs()):
             s = cfg.layer_specs[li]
+            self.shift_states.append(
+                torch.zeros(state_slots, cfg.hidden_size, dtype=torch.float32, device=device)
+                if s.shift else None)
+            if s.kind == "talk_attention":
+                if s.kv_from >= 0:
+                    e = self.entries[run_of[s.kv_from]]
+                else:
+                    e = (torch.zeros(rows, s.kv_heads * s.dim, dtype=dtype, device=device),
+                         torch.zeros(rows, s.kv_heads * s.vdim, dtype=dtype, device=device))
+                run_of[li] = ri
+                self.entries.append(e)
+                continue
+            run_of[li] = ri
             if s.kind == "attention":
                 e = (torch.zeros(rows, s.kv_heads * s.dim, dtype=dtype, device=device),
                      torch.zeros(rows, s.kv_heads * s.dim, dtype=dtype, device=device))
@@ -124,7 +145,9 @@ class HybridCache:
 
     @property
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for e in self.entries for t in e)
+        own = {t.data_ptr(): t for e in self.entries for t in e}
+        own.update({t.data_ptr(): t for t in self.shift_states if t is not None})
+        return sum(t.numel() * t.element_size() for t in own.values())
 
     @property
     def capacity_tokens(self) -> int:

@@ -20,8 +20,16 @@ class LayerSpec:
 
     kinds: ``attention`` (windowed softmax attention, values = the un-normed keys, linear
     distance bias, head mixing, output gate), ``hgrn2`` (gated linear recurrence with a
-    [dim, vdim] state per head) and ``latent_attention`` (keys / values expanded from a cached
-    low-rank latent plus one shared rotated key)."""
+    [dim, vdim] state per head), ``latent_attention`` (keys / values expanded from a cached
+    low-rank latent plus one shared rotated key) and ``talk_attention`` (biased q / k / v
+    projections, unit-RMS queries and keys, scores mixed across heads before the softmax,
+    attention inside blocks of ``chunk`` positions, optionally the cache of layer ``kv_from``).
+
+    feed-forward kinds (``ff_kind``): ``gated_gelu`` (down(gelu(gate) * up)), ``gelu``
+    (down(gelu(up))) and ``moe`` (``experts`` gated-SiLU experts of width ``ff`` plus
+    ``identity`` pass-through experts, ``top`` per token chosen by softmax score + a learned
+    correction and weighted by the un-renormalised score, and a shared expert of width
+    ``shared_ff`` behind a per-token sigmoid gate)."""
     kind: str
     heads: int
     dim: int
@@ -34,16 +42,27 @@ class LayerSpec:
     rot_dims: int = 0         # how many of the rot_dim dims actually rotate
     rot_base: float = 10000.0
     ff: int = 0
+    chunk: int = 0            # > 0: position i sees j only when i // chunk == j // chunk
+    kv_from: int = -1         # >= 0: keys / values are those of that layer (no own projections)
+    shift: bool = False       # the mixer reads h + (h_prev - h) * mu (token shift)
+    ff_kind: str = "gated_gelu"
+    experts: int = 0
+    identity: int = 0
+    top: int = 0
+    shared_ff: int = 0
 
     @property
     def has_state(self) -> bool:
-        return self.kind == "hgrn2"
+        """The layer keeps something per sequence besides cache rows: a recurrent state, or
+        the previous token's mixer input."""
+        return self.kind == "hgrn2" or self.shift
 
 
 @dataclass(frozen=True)
 class ModelConfig:
     name: str
-    arch: str                 # "llama" (llama / mixtral family), "gpt2" or "buborax" (hybrid)
+    arch: str                 # "llama" (llama / mixtral family), "gpt2", or a hybrid
+                              # (layer-list) design: "buborax", "pulunex"
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -68,6 +87,10 @@ class ModelConfig:
     loop: tuple = ()
     norm_groups: int = 1
     residual_mult: float = 1.0
+    embed_scale: float = 1.0      # the embedding row is multiplied by this
+    logit_scale: float = 1.0      # the LM head's output is multiplied by this
+    learned_pos: bool = False     # a learned vector per position is added to the embedding
+    scalar_norm: bool = False     # every norm's weight is one number (checkpoint layout)
 
     @property
     def is_hybrid(self) -> bool:
@@ -154,6 +177,8 @@ class ModelConfig:
             return 2 * s.kv_heads * s.dim           # normed keys + raw keys (the values)
         if s.kind == "latent_attention":
             return s.kv_rank + s.rot_dim
+        if s.kind == "talk_attention":
+            return 0 if s.kv_from >= 0 else s.kv_heads * (s.dim + s.vdim)
         return 0
 
     def to_dict(self) -> dict:
@@ -216,18 +241,19 @@ GPT2_TINY = replace(GPT2, name="gpt2-tiny", hidden_size=256, num_layers=2, num_h
                     max_position=256, bos_token_id=1023, eos_token_id=1023)
 
 def hybrid_config(name: str, width: int, vocab: int, layer_specs, loop=(), norm_groups: int = 1,
-                  norm_eps: float = 1e-6, residual_mult: float = 1.0) -> ModelConfig:
+                  norm_eps: float = 1e-6, residual_mult: float = 1.0, arch: str = "buborax",
+                  max_position: int = 1 << 20, **extra) -> ModelConfig:
     """A hybrid (layer-list) ModelConfig; the llama-shaped fields hold the widest layer's sizes
     (they only feed capacity estimates)."""
     specs = tuple(layer_specs)
     heads = max(s.heads for s in specs)
     return ModelConfig(
-        name=name, arch="buborax", hidden_size=width, num_layers=len(specs), num_heads=heads,
+        name=name, arch=arch, hidden_size=width, num_layers=len(specs), num_heads=heads,
         num_kv_heads=max(max(s.kv_heads, 1) for s in specs), head_dim=max(s.dim for s in specs),
-        intermediate_size=max(s.ff for s in specs), vocab_size=vocab, max_position=1 << 20,
+        intermediate_size=max(s.ff for s in specs), vocab_size=vocab, max_position=max_position,
         rope_theta=0.0, norm_eps=norm_eps, bos_token_id=0, eos_token_id=-1,
         layer_specs=specs, loop=tuple(loop), norm_groups=norm_groups,
-        residual_mult=residual_mult)
+        residual_mult=residual_mult, **extra)
 
 
 # Buborax at test size: every mixer kind, a loop over two layers, grouped norm, GQA in the
@@ -242,9 +268,23 @@ BUBORAX_TINY = hybrid_config(
         LayerSpec("hgrn2", heads=4, dim=16, vdim=32, ff=160)),
     loop=(1, 3, 2), norm_groups=2, norm_eps=1e-6, residual_mult=0.8)
 
+
+def _pulunex_layer(ff_kind: str, kv_from: int = -1) -> LayerSpec:
+    moe = dict(ff=64, experts=6, identity=2, top=2, shared_ff=96) if ff_kind == "moe" else dict(ff=256)
+    return LayerSpec("talk_attention", heads=4, kv_heads=2, dim=32, vdim=48, scale=0.125,
+                     chunk=40, kv_from=kv_from, shift=True, ff_kind=ff_kind, **moe)
+
+
+# Pulunex at test size: a dense layer, routed layers with identity experts and a shared
+# expert, and a layer that attends another layer's keys and values
+PULUNEX_TINY = hybrid_config(
+    "pulunex-tiny", width=128, vocab=384, arch="pulunex", max_position=1024,
+    layer_specs=(_pulunex_layer("gelu"), _pulunex_layer("moe"), _pulunex_layer("moe", kv_from=1)),
+    norm_eps=1e-6, embed_scale=8.0, logit_scale=0.5, learned_pos=True, scalar_norm=True)
+
 _REGISTRY = {c.name: c for c in
              (GPT2, LLAMA3_8B, LLAMA3_70B, MIXTRAL_8X7B, LLAMA_TINY, LLAMA_TINY128,
-              LLAMA_TINY8, MIXTRAL_TINY, MIXTRAL_TINY8E, GPT2_TINY, BUBORAX_TINY)}
+              LLAMA_TINY8, MIXTRAL_TINY, MIXTRAL_TINY8E, GPT2_TINY, BUBORAX_TINY, PULUNEX_TINY)}
 
 _ALIASES = {
     "openai-community/gpt2": "gpt2",

@@ -25,7 +25,7 @@ from typing import Dict, Iterable, Iterator, Optional, Tuple
 import torch
 
 from .configs import ModelConfig
-from .weights import from_buborax_state_dict, from_hf_state_dict
+from .weights import from_buborax_state_dict, from_hf_state_dict, from_pulunex_state_dict
 
 
 def is_hf_dir(d) -> bool:
@@ -58,7 +58,7 @@ def find_hf_dir(root: str, name: str) -> Optional[Path]:
     return None
 
 
-NATIVE_ARCHS = ("Buborax",)
+NATIVE_ARCHS = ("Buborax", "Pulunex")
 
 
 def buborax_config(c: dict, name: Optional[str] = None) -> ModelConfig:
@@ -106,11 +106,67 @@ def buborax_config(c: dict, name: Optional[str] = None) -> ModelConfig:
                          float(norm.get("eps", 1e-6)), float(c.get("residual_mult", 1.0)))
 
 
+def pulunex_config(c: dict, name: Optional[str] = None) -> ModelConfig:
+    """A Pulunex ``config.json``: ``width``, ``vocab``, ``max_positions``, ``embedding``
+    {scale}, ``logit_scale``, ``norm`` {eps} and ``layers``, a list of {type, mixer {heads,
+    kv_heads, dim, vdim, scale, mask {size}, kv_from}, mlp} with mlp null, {kind: dense, ff} or
+    {kind: moe, expert {ff}, router {experts, identity, top}, shared {ff}}. Every size and
+    constant is read from it."""
+    from .configs import LayerSpec, hybrid_config
+    specs = []
+    for i, L in enumerate(c["layers"]):
+        mx, kind = L["mixer"], L["type"]
+        if kind != "attention":
+            raise ValueError(f"unsupported mixer type '{kind}'")
+        H, d = int(mx["heads"]), int(mx["dim"])
+        G = int(mx.get("kv_heads") or H)
+        if H % G:
+            raise ValueError("attention: heads must be a multiple of kv_heads")
+        src = mx.get("kv_from")
+        src = -1 if src is None else int(src)
+        if src >= 0:
+            o = specs[src] if src < i else None
+            if o is None or o.kv_from >= 0 or (o.kv_heads, o.dim, o.vdim) != (
+                    G, d, int(mx.get("vdim", d))):
+                raise ValueError(f"layer {i}: kv_from {src} must name an earlier layer with "
+                                 "projections of its own and the same key / value sizes")
+        ff = dict(ff=0)
+        mlp = L.get("mlp")
+        if mlp:
+            fk = mlp.get("kind", "dense")
+            if fk == "dense":
+                ff = dict(ff=int(mlp["ff"]), ff_kind="gelu")
+            elif fk == "moe":
+                r = mlp["router"]
+                ff = dict(ff=int(mlp["expert"]["ff"]), ff_kind="moe", experts=int(r["experts"]),
+                          identity=int(r.get("identity") or 0), top=int(r["top"]),
+                          shared_ff=int((mlp.get("shared") or {}).get("ff") or 0))
+                if not 1 <= ff["top"] <= ff["experts"] + ff["identity"]:
+                    raise ValueError(f"layer {i}: router.top {ff['top']} of "
+                                     f"{ff['experts'] + ff['identity']} experts")
+            else:
+                raise ValueError(f"unsupported feed-forward kind '{fk}'")
+        specs.append(LayerSpec("talk_attention", heads=H, kv_heads=G, dim=d,
+                               vdim=int(mx.get("vdim", d)),
+                               scale=float(mx.get("scale", d ** -0.5)),
+                               chunk=int((mx.get("mask") or {}).get("size") or 0), kv_from=src,
+                               shift=True, **ff))
+    norm = c.get("norm") or {}
+    return hybrid_config(name or c.get("_name_or_path") or "pulunex", int(c["width"]),
+                         int(c["vocab"]), specs, norm_eps=float(norm.get("eps", 1e-6)),
+                         arch="pulunex", max_position=int(c["max_positions"]),
+                         embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                         logit_scale=float(c.get("logit_scale", 1.0)), learned_pos=True,
+                         scalar_norm=True)
+
+
 def config_from_hf(c: dict, name: Optional[str] = None) -> ModelConfig:
     """Map a ``config.json``: HF llama / mistral / mixtral / gpt2 model types, or one of the
-    native layer-list designs (``architecture``: Buborax)."""
+    native layer-list designs (``architecture``: Buborax, Pulunex)."""
     if c.get("architecture") == "Buborax":
         return buborax_config(c, name)
+    if c.get("architecture") == "Pulunex":
+        return pulunex_config(c, name)
     mt = c.get("model_type", "")
     name = name or c.get("_name_or_path") or mt
     if mt == "gpt2":
@@ -220,7 +276,9 @@ def load_hf_dir(d, device="cpu", dtype=torch.bfloat16, name: Optional[str] = Non
     cfg = config_from_hf(json.loads((d / "config.json").read_text()), name)
     sd = LazyStateDict(d)
     try:
-        if cfg.is_hybrid:
+        if cfg.arch == "pulunex":
+            params = from_pulunex_state_dict(cfg, sd, dtype=dtype)
+        elif cfg.is_hybrid:
             params = from_buborax_state_dict(cfg, sd, dtype=dtype)
         else:
             params = from_hf_state_dict(cfg, sd, layers=layers, first=first, last=last,

@@ -1,5 +1,6 @@
-"""Hybrid decoder (arch ``buborax``): a layer list that mixes windowed attention, latent
-attention and a gated linear recurrence, with a shared-weight loop, grouped RMS norms and an
+"""Hybrid decoder (archs ``buborax``, ``pulunex``): a layer list that mixes windowed attention,
+latent attention, a gated linear recurrence and block attention with head-mixed scores; dense,
+gated and routed feed-forwards; a shared-weight loop, grouped RMS norms, token shift and an
 fp32 residual stream — served by the same engine, scheduler, block manager and runner as the
 transformer families.
 
@@ -25,7 +26,7 @@ import torch
 from ..engine.batch import DeviceBatch
 from ..ops import hybrid as H
 from .configs import ModelConfig
-from .mixers import MIXERS, StepView, derive_constants
+from .mixers import FEED_FORWARDS, MIXERS, StepView, derive_constants
 from .model import TransformerLM
 
 
@@ -72,7 +73,10 @@ class HybridLM(TransformerLM):
 
     # ------------------------------------------------------------------ forward
     def embed(self, b: DeviceBatch) -> torch.Tensor:
-        return H.embedding_f32(b.input_ids, self.params["embed"])[0]
+        cfg, p = self.cfg, self.params
+        return H.embedding_f32(b.input_ids, p["embed"], scale=cfg.embed_scale,
+                               pos_table=p.get("pos_embed") if cfg.learned_pos else None,
+                               positions=b.positions)[0]
 
     def forward_layers(self, x: torch.Tensor, b: DeviceBatch, kv_caches) -> torch.Tensor:
         cfg, p = self.cfg, self.params
@@ -89,14 +93,17 @@ class HybridLM(TransformerLM):
                     pending = None
                 y = H.linear_any(H.concat_cast(x, x0, self.dtype), p["loop_in"])
                 h = H.resadd_groupnorm(x, y, lp["norm1"], groups, eps, mult=1.0, keep=0.0,
-                                       bias=p["loop_step"][t])
+                                       bias=p["loop_step"][t], out_f32=spec.shift)
             else:
-                h = H.resadd_groupnorm(x, pending, lp["norm1"], groups, eps, mult=m)
+                h = H.resadd_groupnorm(x, pending, lp["norm1"], groups, eps, mult=m,
+                                       out_f32=spec.shift)
+            if spec.shift:                  # the mixer reads the rows mixed with their predecessors
+                h = H.token_shift(h, lp["shift"], kv_caches.shift_states[ri], step.state_slots,
+                                  step.cu_seqlens, step.max_seqlen, step.positions)
             y = MIXERS[spec.kind](spec, lp, h, step, entries[ri], eps)
             if spec.ff:
                 h = H.resadd_groupnorm(x, y, lp["norm2"], groups, eps, mult=m)
-                act = H.gelu_mul(H.linear_any(h, lp["w_gu"]), spec.ff, self.dtype)
-                y = H.linear_any(act, lp["w_down"])
+                y = FEED_FORWARDS[spec.ff_kind](spec, lp, h)
             pending = y
             if self.layer_trace is not None:
                 H.resadd_groupnorm(x, pending, None, groups, eps, mult=m)
@@ -114,8 +121,10 @@ class HybridLM(TransformerLM):
             rows = b.last_token_idx
         else:
             return H.resadd_groupnorm(hidden, None, p["final_norm"], cfg.norm_groups,
-                                      cfg.norm_eps)
-        return H.groupnorm_rows(hidden, rows, p["final_norm"], cfg.norm_groups, cfg.norm_eps)
+                                      cfg.norm_eps, gain=cfg.logit_scale)
+        # the logit scale rides on the final norm's output: the head is linear
+        return H.groupnorm_rows(hidden, rows, p["final_norm"], cfg.norm_groups, cfg.norm_eps,
+                                gain=cfg.logit_scale)
 
     def head_logits(self, h: torch.Tensor) -> torch.Tensor:
         return H.linear_any(h, self.params["lm_head"], out_f32=True)

@@ -44,6 +44,10 @@ def derive_constants(spec: LayerSpec, lp: dict, device) -> None:
     elif spec.kind == "latent_attention":
         i = torch.arange(spec.rot_dims // 2, dtype=torch.float64)
         lp["inv_freq"] = torch.pow(spec.rot_base, -2.0 * i / max(1, spec.rot_dims)).float().to(device)
+    elif spec.kind == "talk_attention":
+        lp["talk"] = lp["talk"].float().contiguous()
+    if spec.ff_kind == "moe" and spec.ff:
+        lp["correction"] = lp["correction"].float().contiguous()
 
 
 def attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
@@ -94,5 +98,44 @@ def latent_attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, 
     return H.linear_any(o.view(T, Hh * dv), lp["wo"])
 
 
+def talk_attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
+    """Softmax attention inside blocks of ``spec.chunk`` positions: biased q / k / v, unit-RMS
+    q and k, the heads' scores mixed by ``talk`` before the softmax. The mixing is folded into
+    the queries (``ops.hybrid.talk_prepare``), so the attention itself is the plain kernel with
+    one key head spanning the cached row and G value heads. ``cache`` may be another layer's
+    (``spec.kv_from``): then only queries are projected."""
+    Hh, G, d, dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    kc, vc = cache
+    proj = H.linear_any(h, lp["w_in"])                       # fp32 [T, q (| k | v)]
+    q = H.talk_prepare(proj, lp["b_in"], lp["talk"], eps, Hh, G, d, dv, kc, vc,
+                       step.slot_mapping, own_kv=spec.kv_from < 0)
+    o = H.window_attention(q, kc, vc, G * d, dv, Hh, G, step.cu_seqlens, step.max_seqlen,
+                           step.positions, step.block_tables, step.block_size,
+                           spec.window or (1 << 30), spec.scale, chunk=spec.chunk, k_groups=1)
+    return H.linear_any(o, lp["wo"])
+
+
 MIXERS = {"attention": attention_mixer, "hgrn2": hgrn2_mixer,
-          "latent_attention": latent_attention_mixer}
+          "latent_attention": latent_attention_mixer, "talk_attention": talk_attention_mixer}
+
+
+# ----------------------------------------------------------------------------- feed-forwards
+def gated_gelu_ff(spec: LayerSpec, lp: dict, h):
+    act = H.act_mul(H.linear_any(h, lp["w_gu"]), spec.ff, h.dtype, "gelu_mul")
+    return H.linear_any(act, lp["w_down"])
+
+
+def gelu_ff(spec: LayerSpec, lp: dict, h):
+    act = H.act_mul(H.linear_any(h, lp["w_up"]), spec.ff, h.dtype, "gelu")
+    return H.linear_any(act, lp["w_down"])
+
+
+def moe_ff(spec: LayerSpec, lp: dict, h):
+    """Routed gated-SiLU experts + identity experts + a gated shared expert, summed in fp32."""
+    ng = 1 if spec.shared_ff else 0
+    tw, ti, gates = H.score_router(h, lp["router"], lp["correction"], spec.top, ng)
+    shared = (lp["ws_gu"], lp["ws_down"], gates) if ng else None
+    return H.moe_experts_f32(h, lp["w_gu"], lp["w_down"], tw, ti, shared)
+
+
+FEED_FORWARDS = {"gated_gelu": gated_gelu_ff, "gelu": gelu_ff, "moe": moe_ff}

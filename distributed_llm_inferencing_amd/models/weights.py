@@ -37,7 +37,15 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
       latent_attention: w_in [H*(d+dr) + r + dr, D] = q | compressed kv, c_norm [r],
                         w_ukT [H, r, d] (per head, transposed: the absorb projection),
                         w_uv [H, dv, r], wo [D, H*dv]
-      feed-forward:     norm2 [D], w_gu [2F, D] = gate | up, w_down [D, F]"""
+      talk_attention:   shift [D], w_in [(H*d + G*d + G*dv), D] = q | k | v with b_in (a layer
+                        that attends another layer's cache holds the q part only),
+                        talk [H, H] fp32, wo [D, H*dv]
+      feed-forward:     norm2 [D], then by ``ff_kind``
+        gated_gelu:     w_gu [2F, D] = gate | up, w_down [D, F]
+        gelu:           w_up [F, D], w_down [D, F]
+        moe:            router [E + I (+ 1), D] (the last row is the shared expert's gate),
+                        correction [E + I] fp32, w_gu [E, 2F, D] = gate | up per expert,
+                        w_down [E, D, F], shared expert ws_gu [2Fs, D], ws_down [D, Fs]"""
     D = cfg.hidden_size
     s = cfg.layer_specs[i]
     p = f"layers.{i}."
@@ -53,10 +61,25 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
         out.update({p + "w_in": (H * (d + s.rot_dim) + s.kv_rank + s.rot_dim, D),
                     p + "c_norm": (s.kv_rank,), p + "w_ukT": (H, s.kv_rank, d),
                     p + "w_uv": (H, dv, s.kv_rank), p + "wo": (D, H * dv)})
+    elif s.kind == "talk_attention":
+        n_in = H * d + (0 if s.kv_from >= 0 else s.kv_heads * (d + dv))
+        out.update({p + "shift": (D,), p + "w_in": (n_in, D), p + "b_in": (n_in,),
+                    p + "talk": (H, H), p + "wo": (D, H * dv)})
     else:
         raise ValueError(f"unknown mixer kind '{s.kind}'")
-    if s.ff:
+    if s.ff and s.ff_kind == "gated_gelu":
         out.update({p + "norm2": (D,), p + "w_gu": (2 * s.ff, D), p + "w_down": (D, s.ff)})
+    elif s.ff and s.ff_kind == "gelu":
+        out.update({p + "norm2": (D,), p + "w_up": (s.ff, D), p + "w_down": (D, s.ff)})
+    elif s.ff and s.ff_kind == "moe":
+        n = s.experts + s.identity
+        out.update({p + "norm2": (D,), p + "router": (n + (1 if s.shared_ff else 0), D),
+                    p + "correction": (n,), p + "w_gu": (s.experts, 2 * s.ff, D),
+                    p + "w_down": (s.experts, D, s.ff)})
+        if s.shared_ff:
+            out.update({p + "ws_gu": (2 * s.shared_ff, D), p + "ws_down": (D, s.shared_ff)})
+    elif s.ff:
+        raise ValueError(f"unknown feed-forward kind '{s.ff_kind}'")
     return out
 
 
@@ -88,6 +111,8 @@ def global_param_shapes(cfg: ModelConfig, first: bool, last: bool) -> Dict[str, 
         s.update({"embed": (v, d), "final_norm": (d,), "lm_head": (v, d)})
         if cfg.loop:
             s.update({"loop_in": (d, 2 * d), "loop_step": (cfg.loop[2], d)})
+        if cfg.learned_pos:
+            s["pos_embed"] = (cfg.max_position, d)
         return s
     if first or (last and cfg.tie_embeddings):
         s["embed"] = (v, d)
@@ -159,6 +184,12 @@ def _hybrid_init(name: str, shape: tuple, dev, dtype, seed: int) -> torch.Tensor
     if name.endswith(".talk"):
         t = torch.eye(shape[0]) + 0.2 * torch.randn(shape, generator=g)
         return t.to(dev, torch.float32)
+    if name.endswith(".correction"):
+        return (0.05 * torch.randn(shape, generator=g)).to(dev, torch.float32)
+    if name.endswith(".shift"):
+        return torch.rand(shape, generator=g).to(dev, dtype)
+    if name.endswith(".b_in"):
+        return (0.2 * torch.randn(shape, generator=g)).to(dev, dtype)
     if name.endswith(".lower"):
         return (0.9 * torch.rand(shape, generator=g)).to(dev, dtype)
     if name.endswith((".f_b", "loop_step")):
@@ -302,4 +333,46 @@ def from_buborax_state_dict(cfg: ModelConfig, sd, dtype=torch.bfloat16) -> Dict[
             out[p + "norm2"] = cv(sd[a + "norm2"])
             out[p + "w_gu"] = cv(torch.cat([sd[a + "mlp.gate"], sd[a + "mlp.up"]], 0))
             out[p + "w_down"] = cv(sd[a + "mlp.down"])
+    return out
+
+
+# ----------------------------------------------------------------------------- Pulunex files
+def from_pulunex_state_dict(cfg: ModelConfig, sd, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Convert a Pulunex checkpoint (tensor names ``embed``, ``pos``, ``head``, ``final.norm``,
+    ``l<i>.norm1|norm2|shift``, ``l<i>.mix.q|k|v`` with ``.b`` biases, ``l<i>.mix.talk|o``,
+    ``l<i>.mlp.up|down`` or ``l<i>.mlp.router|correction|e<j>.gate|up|down|shared.*``; linear
+    weights [out, in], norm weights single numbers) into ``hybrid_layer_shapes``' layout: a
+    norm's number becomes a constant vector, projections that read the same input are stacked,
+    the experts are stacked, and the shared expert's gate row is appended to the router."""
+    D = cfg.hidden_size
+    cv = lambda t: t.detach().to(dtype).contiguous()  # noqa: E731
+    vec = lambda t: t.detach().to(dtype).reshape(1).expand(D).contiguous()  # noqa: E731
+    out = {"embed": cv(sd["embed"]), "pos_embed": cv(sd["pos"]), "lm_head": cv(sd["head"]),
+           "final_norm": vec(sd["final.norm"])}
+    for i, s in enumerate(cfg.layer_specs):
+        a, p = f"l{i}.", f"layers.{i}."
+        m = a + "mix."
+        out[p + "norm1"] = vec(sd[a + "norm1"])
+        out[p + "shift"] = cv(sd[a + "shift"])
+        parts = ["q"] if s.kv_from >= 0 else ["q", "k", "v"]
+        out[p + "w_in"] = cv(torch.cat([sd[m + n] for n in parts], 0))
+        out[p + "b_in"] = cv(torch.cat([sd[m + n + ".b"] for n in parts], 0))
+        out[p + "talk"] = sd[m + "talk"].detach().float().contiguous()
+        out[p + "wo"] = cv(sd[m + "o"])
+        if not s.ff:
+            continue
+        f = a + "mlp."
+        out[p + "norm2"] = vec(sd[a + "norm2"])
+        if s.ff_kind == "gelu":
+            out[p + "w_up"], out[p + "w_down"] = cv(sd[f + "up"]), cv(sd[f + "down"])
+            continue
+        rows = [sd[f + "router"]] + ([sd[f + "shared.sg"].reshape(1, D)] if s.shared_ff else [])
+        out[p + "router"] = cv(torch.cat(rows, 0))
+        out[p + "correction"] = sd[f + "correction"].detach().float().contiguous()
+        out[p + "w_gu"] = cv(torch.stack([torch.cat([sd[f"{f}e{e}.gate"], sd[f"{f}e{e}.up"]], 0)
+                                          for e in range(s.experts)]))
+        out[p + "w_down"] = cv(torch.stack([sd[f"{f}e{e}.down"] for e in range(s.experts)]))
+        if s.shared_ff:
+            out[p + "ws_gu"] = cv(torch.cat([sd[f + "shared.gate"], sd[f + "shared.up"]], 0))
+            out[p + "ws_down"] = cv(sd[f + "shared.down"])
     return out

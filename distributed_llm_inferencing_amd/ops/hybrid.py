@@ -86,24 +86,32 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Te
 
 
 # ----------------------------------------------------------------------------- rows
-def embedding_f32(ids: torch.Tensor, table: torch.Tensor, copy: bool = False):
-    """fp32 rows of ``table`` (and a second copy when asked: the loop input)."""
+def embedding_f32(ids: torch.Tensor, table: torch.Tensor, copy: bool = False,
+                  scale: float = 1.0, pos_table: Optional[torch.Tensor] = None,
+                  positions: Optional[torch.Tensor] = None):
+    """fp32 rows of ``table`` times ``scale``, plus the row ``positions[t]`` of ``pos_table``
+    when given (and a second copy when asked: the loop input)."""
     if not table.is_cuda:
-        x = table[ids.long()].float()
+        x = table[ids.long()].float() * scale
+        if pos_table is not None:
+            x = x + pos_table[positions.long()].float()
         return (x, x.clone()) if copy else (x, None)
     T, D = ids.shape[0], table.shape[1]
     x = torch.empty(T, D, dtype=torch.float32, device=table.device)
     x0 = torch.empty_like(x) if copy else None
     _call("dli_embedding_f32", _p(x), _p(x0), _p(ids), _p(table), T, D, table.shape[0],
-          _dt(table.dtype), _st())
+          float(scale), _p(pos_table), _p(positions),
+          pos_table.shape[0] if pos_table is not None else 0, _dt(table.dtype), _st())
     return x, x0
 
 
 def resadd_groupnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[torch.Tensor],
                      groups: int, eps: float, mult: float = 1.0, keep: float = 1.0,
-                     bias: Optional[torch.Tensor] = None, dtype=None) -> Optional[torch.Tensor]:
+                     bias: Optional[torch.Tensor] = None, dtype=None, gain: float = 1.0,
+                     out_f32: bool = False) -> Optional[torch.Tensor]:
     """In place on the fp32 stream: x = keep * x + mult * y + bias (y, bias optional); returns
-    the grouped RMS norm of the new x times ``w`` in the storage dtype (None when w is None)."""
+    the grouped RMS norm of the new x times ``w`` times ``gain`` in the storage dtype (None when
+    w is None), or unrounded in fp32 with ``out_f32`` (what a token shift reads)."""
     dtype = dtype or (w.dtype if w is not None else torch.bfloat16)
     if not x.is_cuda:
         if keep != 1.0:
@@ -112,25 +120,48 @@ def resadd_groupnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[tor
             x.add_(y.float(), alpha=mult)
         if bias is not None:
             x.add_(bias.float())
-        return None if w is None else R.group_rmsnorm(x, w, groups, eps, dtype)
+        if w is None:
+            return None
+        h = R.group_rmsnorm(x, w, groups, eps, torch.float32)
+        if gain != 1.0:
+            h = h * gain
+        return h if out_f32 else h.to(dtype)
     rows, dim = x.shape
-    h = torch.empty(rows, dim, dtype=dtype, device=x.device) if w is not None else None
+    h = (torch.empty(rows, dim, dtype=torch.float32 if out_f32 else dtype, device=x.device)
+         if w is not None else None)
     _call("dli_resadd_groupnorm", _p(x), _p(y), y.stride(0) if y is not None else 0, _p(bias),
           float(keep), float(mult), _p(w), _p(h), dim, rows, dim, groups, float(eps), None,
-          _dt(dtype), _st())
+          float(gain), int(out_f32), _dt(dtype), _st())
     return h
 
 
 def groupnorm_rows(x: torch.Tensor, rows_idx: torch.Tensor, w: torch.Tensor, groups: int,
-                   eps: float) -> torch.Tensor:
-    """Grouped RMS norm of the rows ``rows_idx`` (int64) of the fp32 stream."""
+                   eps: float, gain: float = 1.0) -> torch.Tensor:
+    """Grouped RMS norm (times ``gain``) of the rows ``rows_idx`` (int64) of the fp32 stream."""
     if not x.is_cuda:
-        return R.group_rmsnorm(x.index_select(0, rows_idx), w, groups, eps, w.dtype)
+        h = R.group_rmsnorm(x.index_select(0, rows_idx), w, groups, eps, torch.float32)
+        return (h * gain if gain != 1.0 else h).to(w.dtype)
     n, dim = rows_idx.shape[0], x.shape[1]
     h = torch.empty(n, dim, dtype=w.dtype, device=x.device)
     _call("dli_resadd_groupnorm", _p(x), None, 0, None, 1.0, 1.0, _p(w), _p(h), dim, n, dim,
-          groups, float(eps), _p(rows_idx), _dt(w.dtype), _st())
+          groups, float(eps), _p(rows_idx), float(gain), 0, _dt(w.dtype), _st())
     return h
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, slots: torch.Tensor,
+                cu_seqlens: torch.Tensor, max_seqlen: int, positions: torch.Tensor) -> torch.Tensor:
+    """Token shift of the normed rows h (fp32 [T, D]): u_t = h_t + (h_{t-1} - h_t) * mu, in the
+    storage dtype of ``mu``. h_{t-1} of a portion's first row comes from the sequence's slot
+    of ``state`` (fp32 [slots, D]; zeros at position 0), which then receives the portion's
+    last row."""
+    if not h.is_cuda:
+        return R.token_shift(h, mu, state, slots, cu_seqlens, positions, mu.dtype)
+    T, D = h.shape
+    S = cu_seqlens.shape[0] - 1
+    out = torch.empty(T, D, dtype=mu.dtype, device=h.device)
+    _call("dli_token_shift", _p(h), _p(mu), _p(state), _p(slots), _p(cu_seqlens), _p(positions),
+          _p(out), S, int(max_seqlen), D, _dt(mu.dtype), _st())
+    return out
 
 
 def concat_cast(a: torch.Tensor, b: torch.Tensor, dtype) -> torch.Tensor:
@@ -143,14 +174,26 @@ def concat_cast(a: torch.Tensor, b: torch.Tensor, dtype) -> torch.Tensor:
     return out
 
 
-def gelu_mul(gu: torch.Tensor, F_: int, dtype) -> torch.Tensor:
-    """gelu_tanh(gu[:, :F]) * gu[:, F:2F] for an fp32 [T, 2F] projection."""
+_ACT_KINDS = {"gelu_mul": 0, "silu_mul": 1, "gelu": 2}
+
+
+def act_mul(gu: torch.Tensor, F_: int, dtype, kind: str = "gelu_mul",
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The feed-forward's middle for an fp32 projection: ``gelu_mul`` / ``silu_mul`` =
+    act(gu[:, :F]) * gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F]). ``rows`` (device int32
+    scalar): only that many leading rows hold data (routed rows of a mixture)."""
     if not gu.is_cuda:
-        return R.gelu_mul(gu, F_, dtype)
+        return R.act_mul(gu, F_, dtype, kind)
     T = gu.shape[0]
     out = torch.empty(T, F_, dtype=dtype, device=gu.device)
-    _call("dli_gelu_mul", _p(out), F_, _p(gu), gu.stride(0), T, F_, _dt(dtype), _st())
+    _call("dli_act_mul", _p(out), F_, _p(gu), gu.stride(0), T, F_, _ACT_KINDS[kind], _p(rows),
+          _dt(dtype), _st())
     return out
+
+
+def gelu_mul(gu: torch.Tensor, F_: int, dtype) -> torch.Tensor:
+    """gelu_tanh(gu[:, :F]) * gu[:, F:2F] for an fp32 [T, 2F] projection."""
+    return act_mul(gu, F_, dtype, "gelu_mul")
 
 
 # ----------------------------------------------------------------------------- mixers
@@ -162,6 +205,23 @@ def attn_prepare(proj, qw, kw, eps, H, G, d, kcache, vcache, slots):
     q = torch.empty(T, H * d, dtype=dtype, device=proj.device)
     _call("dli_attn_prepare", _p(proj), proj.stride(0), _p(qw), _p(kw), float(eps), T, H, G, d,
           _p(q), _p(kcache), _p(vcache), _p(slots), _dt(dtype), _st())
+    return q
+
+
+def talk_prepare(proj, bias, talk, eps, H, G, d, dv, kcache, vcache, slots, own_kv: bool):
+    """q / k / v of an attention whose scores are mixed across heads before the softmax (see
+    ``reference.talk_prepare``): adds the projection bias, divides q and k heads by their RMS,
+    writes k and v to the cache rows (``own_kv``), and returns the mixed queries
+    [T, H * G*d] in the storage dtype: head h scores whole key rows."""
+    dtype = bias.dtype
+    if not proj.is_cuda:
+        return R.talk_prepare(proj, bias, talk, eps, H, G, d, dv, kcache, vcache, slots, own_kv,
+                              dtype)
+    T = proj.shape[0]
+    q = torch.empty(T, H * G * d, dtype=dtype, device=proj.device)
+    _call("dli_talk_prepare", _p(proj), proj.stride(0), _p(bias), _p(talk), float(eps), T, H, G,
+          d, dv, _p(q), _p(kcache) if own_kv else None, _p(vcache) if own_kv else None,
+          _p(slots), _dt(dtype), _st())
     return q
 
 
@@ -185,13 +245,18 @@ def mla_prepare(proj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots
 
 
 def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, positions,
-                     block_tables, block_size, window, scale, slopes=None, talk=None, gate=None):
+                     block_tables, block_size, window, scale, slopes=None, talk=None, gate=None,
+                     chunk: int = 0, k_groups: Optional[int] = None):
     """See ``reference.window_attention`` / window_attention.hip. q [T, H*dq] (storage dtype);
-    caches are token-major rows; returns [T, H*dv] in the storage dtype."""
+    caches are token-major rows; returns [T, H*dv] in the storage dtype. ``chunk`` > 0 limits
+    a query to the keys of its own block of that many positions; ``k_groups`` is the number of
+    key heads per cache row when it is not the number of value heads G."""
+    Gk = G if k_groups is None else int(k_groups)
+    chunk = int(chunk)
     if not q.is_cuda:
         return R.window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions,
                                   block_tables, block_size, window, scale, slopes, talk, gate,
-                                  out_dtype=q.dtype)
+                                  out_dtype=q.dtype, chunk=chunk, k_groups=Gk)
     T = q.shape[0]
     S = cu_seqlens.shape[0] - 1
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
@@ -203,15 +268,15 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
         rowhead = int(G == 1 and H > 1 and int(max_seqlen) == 1 and talk is None and gate is None
                       and slopes is None and q.stride(0) == H * dq)
         nb = lib.dli_window_attention_mfma_workspace_bytes(S, int(max_seqlen), T, H, dv,
-                                                           int(window), int(talk is not None),
-                                                           rowhead)
+                                                           int(min(window, chunk) if chunk else window),
+                                                           int(talk is not None), rowhead)
         ws = _gemm.workspace(q.device, nb) if nb else None       # key-split form (decode steps)
         rc = lib.dli_window_attention_mfma(
             _p(q), q.stride(0), _p(k_cache), k_cache.stride(0), _p(v_cache), v_cache.stride(0),
             _p(out), out.stride(0), _p(gate), gate.stride(0) if gate is not None else 0,
             _p(slopes), _p(talk), _p(cu_seqlens), _p(positions), _p(block_tables),
             block_tables.stride(0), block_size, S, int(max_seqlen), H, G, dq, dv, int(window),
-            float(scale), T, _p(ws), rowhead, _st())
+            float(scale), T, _p(ws), rowhead, Gk, chunk, _st())
         if rc == 0:
             return out
         if rc != _NOT_SUPPORTED:
@@ -220,7 +285,8 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
           _p(v_cache), v_cache.stride(0), _p(out), out.stride(0), _p(gate),
           gate.stride(0) if gate is not None else 0, _p(slopes), _p(talk), _p(cu_seqlens),
           _p(positions), _p(block_tables), block_tables.stride(0), block_size, S,
-          int(max_seqlen), H, G, dq, dv, int(window), float(scale), _dt(q.dtype), _st())
+          int(max_seqlen), H, G, dq, dv, int(window), float(scale), Gk, chunk, _dt(q.dtype),
+          _st())
     return out
 
 
@@ -236,4 +302,64 @@ def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, max_seqlen
     _call("dli_hgrn2", _p(proj), proj.stride(0), _p(f_bias), _p(lower), _p(norm_w), float(eps),
           _p(state), _p(slots), _p(cu_seqlens), _p(positions), _p(out), out.stride(0), S,
           int(max_seqlen), H, d, dv, _dt(dtype), _st())
+    return out
+
+
+# ----------------------------------------------------------------------------- mixture of experts
+def score_router(h, w_router, correction, top: int, n_gate: int = 0):
+    """Router with un-renormalised softmax weights and a choice correction (see
+    ``reference.score_router``): (weights fp32 [T, top], ids int32 [T, top], gates fp32
+    [T, n_gate]) from one pass over each token's row, logits in fp32."""
+    if not h.is_cuda:
+        return R.score_router(h, w_router, correction, top, n_gate)
+    T, D = h.shape
+    n = w_router.shape[0] - n_gate
+    w = torch.empty(T, top, dtype=torch.float32, device=h.device)
+    ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
+    gates = torch.empty(T, max(n_gate, 1), dtype=torch.float32, device=h.device)
+    _call("dli_score_router", _p(w), _p(ids), _p(gates), _p(h), h.stride(0), _p(w_router),
+          _p(correction), T, D, n, n_gate, top, _dt(h.dtype), _st())
+    return w, ids, gates[:, :n_gate]
+
+
+def grouped_linear_any(x, w, offsets, src, n: int) -> torch.Tensor:
+    """Per-expert projections of routed rows: out[p] = x[src[p]] @ w[e]^T for the permuted rows
+    p in [offsets[e], offsets[e+1]) (``src`` None: x is already permuted). x [*, K], w
+    [E, N, K], out fp32 [n, N]; rows past offsets[E] are not written."""
+    E, Nn, K = w.shape
+    out = torch.empty(max(n, 1), Nn, dtype=torch.float32, device=x.device)
+    if n > 0:
+        _call("dli_gemm_any_grouped", _p(x), x.stride(0), _p(w), w.stride(1), w.stride(0),
+              _p(out), out.stride(0), n, Nn, K, _dt(x.dtype), E, _p(offsets), _p(src), _st())
+    return out
+
+
+def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None) -> torch.Tensor:
+    """Weighted sum of every token's chosen experts in fp32 (``reference.moe_experts_f32``):
+    ids below E run the gated-SiLU experts as grouped GEMMs over the rows sorted by expert, ids
+    from E on are identity experts; ``shared`` = (ws_gu, ws_down, gate [T]) adds the always-on
+    expert times its gate. No host synchronisation: a captured graph replays it."""
+    if not x.is_cuda:
+        return R.moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared)
+    T, D = x.shape
+    k = topk_ids.shape[1]
+    E, F2, _ = w_gu.shape
+    n = T * k
+    dev = x.device
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    pos = torch.empty(n, dtype=torch.int32, device=dev)
+    src = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
+    _call("dli_moe_align", _p(offsets), _p(pos), _p(src), _p(topk_ids), n, k, 0, E, _st())
+    gu = grouped_linear_any(x, w_gu, offsets, src, n)
+    act = act_mul(gu, F2 // 2, x.dtype, "silu_mul", rows=offsets[E:])
+    y = grouped_linear_any(act, w_down, offsets, None, n)
+    ys = gate = None
+    if shared is not None:
+        ws_gu, ws_down, gate = shared
+        a = act_mul(linear_any(x, ws_gu), ws_gu.shape[0] // 2, x.dtype, "silu_mul")
+        ys = linear_any(a, ws_down)
+    out = torch.empty(T, D, dtype=torch.float32, device=dev)
+    _call("dli_moe_combine_f32", _p(out), _p(y), _p(topk_w), _p(pos), _p(topk_ids), _p(x), x.stride(0),
+          _p(ys), _p(gate), gate.stride(0) if gate is not None else 0, T, k, D, E,
+          _dt(x.dtype), _st())
     return out

@@ -394,6 +394,17 @@ def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
     return (n.reshape(T, D) * w.float()).to(out_dtype)
 
 
+def act_mul(gu: torch.Tensor, F_: int, out_dtype: torch.dtype, kind: str) -> torch.Tensor:
+    """The feed-forward's middle, fp32 in: ``gelu_mul`` / ``silu_mul`` = act(gu[:, :F]) *
+    gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F])."""
+    g = gu[:, :F_].float()
+    if kind == "gelu":
+        return F.gelu(g, approximate="tanh").to(out_dtype)
+    u = gu[:, F_:2 * F_].float()
+    a = F.gelu(g, approximate="tanh") if kind == "gelu_mul" else F.silu(g)
+    return (a * u).to(out_dtype)
+
+
 def gelu_mul(gu: torch.Tensor, F_: int, out_dtype: torch.dtype) -> torch.Tensor:
     """gelu_tanh(gu[:, :F]) * gu[:, F:2F] (plain concatenation, fp32 in)."""
     g, u = gu[:, :F_].float(), gu[:, F_:2 * F_].float()
@@ -449,13 +460,16 @@ def mla_prepare(proj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots
 
 def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions, block_tables,
                      block_size, window, scale, slopes=None, talk=None, gate=None,
-                     out_dtype=None):
+                     out_dtype=None, chunk=0, k_groups=None):
     """q [T, H*dq]; k_cache rows [slots, G*dq]; v_cache rows [slots, >= G*dv] (may be k_cache:
     values = the first dv columns of each kv head's... row when G == 1). Every query at position
     p attends cached positions [max(0, p-window+1), p] of its sequence. fp32 softmax; ``talk``
     [H, H] mixes the heads' normalised weights; ``slopes`` [H] subtract slope*(p-j); ``gate``
-    fp32 [T, H*dv] multiplies the output by its sigmoid."""
+    fp32 [T, H*dv] multiplies the output by its sigmoid. ``chunk`` > 0: only keys of the
+    query's own block of ``chunk`` positions are visible. ``k_groups``: key heads per cache row
+    when it differs from the value heads G (1: every query head scores the whole key row)."""
     T = q.shape[0]
+    Gk = G if k_groups is None else k_groups
     out = torch.zeros(T, H * dv, dtype=torch.float32, device=q.device)
     cu = cu_seqlens.tolist()
     for s in range(len(cu) - 1):
@@ -466,17 +480,19 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions, b
         ctx = int(pos.max()) + 1
         j = torch.arange(ctx, device=q.device)
         sl = (block_tables[s].long()[j // block_size] * block_size + j % block_size)
-        kk = k_cache[sl][:, :G * dq].float().reshape(ctx, G, dq)
+        kk = k_cache[sl][:, :Gk * dq].float().reshape(ctx, Gk, dq)
         vv = v_cache[sl].float()
         vv = torch.stack([vv[:, g * dv:(g + 1) * dv] for g in range(G)], 1)   # [ctx, G, dv]
         qq = q[t0:t1].float().reshape(t1 - t0, H, dq)
         rep = H // G
-        ke = kk.repeat_interleave(rep, dim=1)                                   # [ctx, H, dq]
+        ke = kk.repeat_interleave(H // Gk, dim=1)                               # [ctx, H, dq]
         sc = torch.einsum("thd,jhd->htj", qq, ke) * scale
         dist = (pos[:, None] - j[None, :]).float()                              # [n, ctx]
         if slopes is not None:
             sc = sc - slopes.float()[:, None, None] * dist[None]
         vis = (dist >= 0) & (dist < window)
+        if chunk:
+            vis = vis & ((pos[:, None] // chunk) == (j[None, :] // chunk))
         sc = sc.masked_fill(~vis[None], float("-inf"))
         w = torch.softmax(sc, dim=-1)
         if talk is not None:
@@ -518,3 +534,86 @@ def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, positions,
             out[t0 + t] = o.reshape(H * dv)
         state[sl[s]] = S
     return out.to(out_dtype)
+
+
+def token_shift(h, mu, state, slots, cu_seqlens, positions, out_dtype):
+    """h fp32 [T, D] (normed rows): row t becomes h_t + (h_{t-1} - h_t) * mu, with h_{t-1} the
+    sequence's previous row as it came in — the row before it in this step, the row kept in
+    ``state`` [slots, D] fp32 for a portion's first row, zeros at position 0. The last row of
+    every sequence is kept in ``state``."""
+    out = torch.empty_like(h, dtype=torch.float32)
+    cu, sl = cu_seqlens.tolist(), slots.tolist()
+    m = mu.float()
+    for s in range(len(cu) - 1):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0 or sl[s] < 0:
+            continue
+        hh = h[t0:t1].float()
+        first = (torch.zeros_like(hh[:1]) if int(positions[t0]) == 0
+                 else state[sl[s]].float()[None])
+        prev = torch.cat([first, hh[:-1]], 0)
+        out[t0:t1] = hh + (prev - hh) * m
+        state[sl[s]] = hh[-1]
+    return out.to(out_dtype)
+
+
+def talk_prepare(proj, bias, talk, eps, H, G, d, dv, kcache, vcache, slots, own_kv, out_dtype):
+    """proj fp32 [T, H*d (+ G*d + G*dv)] = [q | k | v] and its bias. q and k heads are divided
+    by their RMS; with ``own_kv`` normed k and v go to the cache rows ``slots``. Returns the
+    queries with the pre-softmax head mixing folded in: since
+        sum_g talk[h, g] (q_g . k_{c(g)}) = sum_c (sum_{g in c} talk[h, g] q_g) . k_c,
+    head h scores the whole cached key row with q'_h [G*d], part c = sum_{g in c} talk[h, g] q_g."""
+    T = proj.shape[0]
+    p = proj.float() + bias.float()
+    q = p[:, :H * d].reshape(T, H, d)
+    qn = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+    if own_kv:
+        k = p[:, H * d:(H + G) * d].reshape(T, G, d)
+        kn = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
+        v = p[:, (H + G) * d:(H + G) * d + G * dv]
+        ok = slots >= 0
+        idx = slots[ok].long()
+        kcache[idx] = kn.reshape(T, G * d)[ok].to(kcache.dtype)
+        vcache[idx] = v[ok].to(vcache.dtype)
+    rep = H // G
+    tk = talk.float().reshape(H, G, rep)                       # [h, c, g in c]
+    qm = torch.einsum("hcr,tcrd->thcd", tk, qn.reshape(T, G, rep, d))
+    return qm.reshape(T, H * G * d).to(out_dtype)
+
+
+def score_router(h, w_router, correction, top, n_gate=0):
+    """Router of a mixture with un-renormalised softmax weights: logits = h @ w_router[:n].T in
+    fp32, s = softmax over all n experts, the ``top`` largest of s + correction are chosen
+    (lowest index on ties), their weights are s. The last ``n_gate`` rows of ``w_router`` are
+    extra gates: sigmoid(h . row). Returns (weights fp32 [T, top], ids int32, gates [T, n_gate])."""
+    n = w_router.shape[0] - n_gate
+    z = h.float() @ w_router.float().t()
+    sc = torch.softmax(z[:, :n], -1)
+    choice = sc + correction.float()
+    ids = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    return sc.gather(1, ids), ids.to(torch.int32), torch.sigmoid(z[:, n:])
+
+
+def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None):
+    """Weighted sum of each token's chosen experts, fp32 out. Expert e < E (w_gu [E, 2F, D] =
+    gate | up, w_down [E, D, F]) is down(silu(gate) * up); ids >= E are identity experts (the
+    input itself). ``shared`` = (ws_gu, ws_down, gate [T]) adds an always-on expert times its
+    per-token gate."""
+    T, D = x.shape
+    E, F2, _ = w_gu.shape
+    out = torch.zeros(T, D, dtype=torch.float32, device=x.device)
+    for e in range(E):
+        rows, slot = (topk_ids == e).nonzero(as_tuple=True)
+        if rows.numel() == 0:
+            continue
+        a = act_mul(linear(x[rows], w_gu[e], out_dtype=torch.float32), F2 // 2, x.dtype, "silu_mul")
+        y = linear(a, w_down[e], out_dtype=torch.float32)
+        out.index_add_(0, rows, y * topk_w[rows, slot][:, None])
+    wi = (topk_w * (topk_ids >= E)).sum(-1, keepdim=True)
+    out += wi * x.float()
+    if shared is not None:
+        ws_gu, ws_down, gate = shared
+        a = act_mul(linear(x, ws_gu, out_dtype=torch.float32), ws_gu.shape[0] // 2, x.dtype,
+                    "silu_mul")
+        out += gate.float().reshape(T, 1) * linear(a, ws_down, out_dtype=torch.float32)
+    return out
