@@ -75,7 +75,8 @@ def block_attention(us, mx, w, pre, eps, kv):
     """us [T, D] mixer inputs of one sequence; kv = (keys, values) to attend. Returns [T, D]."""
     T = us.shape[0]
     H, G, d, dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
-    size, scale = mx["mask"]["size"], mx["scale"]
+    size = (mx.get("mask") or {}).get("size") or max(T, 1)      # no mask: one block
+    scale = mx["scale"]
     kn, v = kv
     q = (us @ w[pre + "q"].T + w[pre + "q.b"]).reshape(T, H, d)
     talk = w[pre + "talk"]
