@@ -46,6 +46,9 @@ struct MfmaArgs {
   const int* block_tables; int bt_stride; int block_size;
   int H, G, dq, dv, window;
   float scale;
+  // Gk: key heads per cache row (the values have G; Gk = 1: every head scores the whole key
+  // row). chunk > 0: a query sees only keys of its own block of `chunk` positions.
+  int Gk, chunk;
   int Hp;        // H rounded up to 32 (mix K dimension)
   int CG;        // kv heads staged per step
   // key-split form (few query tiles, long windows: decode steps): the window's tiles are dealt
@@ -110,11 +113,14 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   const int nq = min(TQ, t_end - t0);
   const int p0 = a.positions[t0 / a.rowmul];      // positions of a portion are consecutive
   const int p_last = a.rowmul > 1 ? p0 : p0 + nq - 1;
-  const int lo = max(0, p0 - a.window + 1);
+  // the first query's lower bound is the lowest of the tile (window and block alike)
+  const int lo = max(max(0, p0 - a.window + 1), a.chunk > 0 ? p0 / a.chunk * a.chunk : 0);
   const int ntiles = (p_last - lo) / TK + 1;
   const int* bt = a.block_tables + (long)s * a.bt_stride;
-  const int hpg = H / G;
+  const int hpg = H / G, Gk = a.Gk, hpk = H / Gk;
   const int my_p = a.rowmul > 1 ? p0 : p0 + fr;   // this lane's query position (column fr)
+  const int my_clo = a.chunk > 0 ? my_p / a.chunk * a.chunk : 0;      // first key of its block
+  const int clo_last = a.chunk > 0 ? p_last / a.chunk * a.chunk : 0;
   const bool my_q = fr < nq;
   const bool has_talk = a.talk != nullptr;
   const int Hp16 = (H + 15) & ~15;
@@ -206,14 +212,14 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
           slot[tid] = j <= p_last ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
         }
       }
-      for (int c0 = 0; c0 < G; c0 += CG) {
-        const int cg = min(CG, G - c0);
+      for (int c0 = 0; c0 < Gk; c0 += CG) {
+        const int cg = min(CG, Gk - c0);
         {                                         // this wave's first head of the step: its
           int h0 = -1;                            // query fragments fly with the K tiles
 #pragma unroll
           for (int h2 = MAXHW - 1; h2 >= 0; --h2) {
             const int hc = wide ? hbase + wave : wave + h2 * NW;
-            if ((!wide || h2 == 0) && hc < H && hc / hpg >= c0 && hc / hpg < c0 + cg) h0 = hc;
+            if ((!wide || h2 == 0) && hc < H && hc / hpk >= c0 && hc / hpk < c0 + cg) h0 = hc;
           }
           qh = h0;
           if (h0 >= 0) load_q(h0, 0, qcur);
@@ -246,7 +252,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         for (int hh = 0; hh < MAXHW; ++hh) {
           const int h = wide ? hbase + wave : wave + hh * NW;
           if (h >= H || (wide && hh)) continue;
-          const int c = h / hpg;
+          const int c = h / hpk;
           if (c < c0 || c >= c0 + cg) continue;
           const u16* kt = Ks + (long)(c - c0) * TK * ldk;
           f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
@@ -256,7 +262,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
 #pragma unroll
           for (int h2 = MAXHW - 1; h2 > hh; --h2) {
             const int hc = wave + h2 * NW;
-            if (!wide && hc < H && hc / hpg >= c0 && hc / hpg < c0 + cg) hn = hc;
+            if (!wide && hc < H && hc / hpk >= c0 && hc / hpk < c0 + cg) hn = hc;
           }
           if (qh != h) load_q(h, 0, qcur);        // not prefetched (first head of the step)
           for (int f0 = 0; f0 < nf; f0 += 4) {
@@ -292,15 +298,17 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
           float sv[8];
           float tmax = -INFINITY;
           // interior tiles (every key visible to every query row): no masking arithmetic
-          const bool interior = nq == TQ && j0 + TK - 1 <= p0 && j0 > p_last - a.window;
+          const bool interior = nq == TQ && j0 + TK - 1 <= p0 && j0 > p_last - a.window &&
+                                j0 >= clo_last;
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               float x = fmaf(sacc[kb][r], scale2, b0 + slope2 * (float)(kb * 16 + r));
               if (!interior) {
-                const int dist = my_p - (j0 + kb * 16 + fq * 4 + r);
-                if (!my_q || dist < 0 || dist >= a.window) x = -INFINITY;
+                const int key = j0 + kb * 16 + fq * 4 + r;
+                const int dist = my_p - key;
+                if (!my_q || dist < 0 || dist >= a.window || key < my_clo) x = -INFINITY;
               }
               sv[kb * 4 + r] = x;
               tmax = fmaxf(tmax, x);
@@ -595,11 +603,12 @@ extern "C" int dli_window_attention_mfma(
     int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int T, void* ws,
     int rowhead, int Gk, int chunk, hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
-  // block masks and key rows whose head count differs from the values' run the scalar form
-  if (chunk != 0 || Gk != G) return (int)hipErrorNotSupported;
+  if (chunk < 0 || Gk < 1) return (int)hipErrorInvalidValue;
+  // keys a query tile can see: bounds the slot table and the key splits
+  const int weff = chunk > 0 && chunk < window ? chunk : window;
   int rowmul = 1;
   if (rowhead) {
-    if (talk != nullptr || gate != nullptr || slopes != nullptr || G != 1 || max_seqlen != 1 ||
+    if (talk != nullptr || gate != nullptr || slopes != nullptr || G != 1 || Gk != 1 || max_seqlen != 1 ||
         ldq != H * dq || ldo != H * dv)
       return (int)hipErrorInvalidValue;
     rowmul = H;            // token t's heads = rows [t*H, (t+1)*H) of a one-head problem
@@ -613,14 +622,14 @@ extern "C" int dli_window_attention_mfma(
                        (uintptr_t)out % 8 == 0 && ldq % 8 == 0 && k_stride % 8 == 0 &&
                        v_stride % 8 == 0 && ldo % 4 == 0;
   const bool wide = talk == nullptr;
-  if (H < 1 || (!wide && H > NW * MAXHW) || G < 1 || H % G || dq % 32 || dv % 16 || !aligned ||
-      window < 1 || block_size < 1)
+  if (H < 1 || (!wide && H > NW * MAXHW) || G < 1 || H % G || H % Gk || dq % 32 || dv % 16 ||
+      !aligned || window < 1 || block_size < 1 || (!wide && Gk != G))
     return (int)hipErrorNotSupported;
   const int dvw = wide ? 512 : 128;
   const int Hp = (H + 31) & ~31, Hp16 = (H + 15) & ~15;
   const int ldk = dq + 16;
   // the whole window's cache rows in LDS when they take at most 16 KB
-  int slot_cap = ((window + TQ - 2) / TK + 2) * TK;
+  int slot_cap = ((weff + TQ - 2) / TK + 2) * TK;
   if ((size_t)slot_cap * 4 > 16 * 1024) slot_cap = 0;
   const size_t fixed = (wide ? (size_t)NW * TQ * 40
                              : (size_t)TQ * TK * (Hp + 8) + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
@@ -629,7 +638,7 @@ extern "C" int dli_window_attention_mfma(
   const size_t budget = 158 * 1024;
   if (fixed + per_cg > budget) return (int)hipErrorNotSupported;
   int CG = (int)((budget - fixed) / per_cg);
-  CG = CG > G ? G : CG;
+  CG = CG > (G > Gk ? G : Gk) ? (G > Gk ? G : Gk) : CG;
   CG = CG > NW ? NW : CG;
   const size_t sh = fixed + CG * per_cg;
   static bool raised = false;
@@ -649,10 +658,10 @@ extern "C" int dli_window_attention_mfma(
   } while (0)
   const int ndvs = (dv + dvw - 1) / dvw, qtiles = (max_seqlen + TQ - 1) / TQ;
   const int nhs = wide ? (H + NW - 1) / NW : 1;
-  const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, H, dv, window, wide) : 1;
+  const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, H, dv, weff, wide) : 1;
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
-             H, G, dq, dv, window, scale, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
+             H, G, dq, dv, window, scale, Gk, chunk, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
              slot_cap, nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);

@@ -104,12 +104,17 @@ def gated_expert(h, w, pre):
     return w[pre + "down"] @ (silu(w[pre + "gate"] @ h) * (w[pre + "up"] @ h))
 
 
-def routed_ff(h, mlp, w, pre):
+def routed_ff(h, mlp, w, pre, margin=None):
+    """``margin`` (a one-element list) is lowered to the gap between the last chosen and the
+    first rejected choice score: how close the routing of this token was to another outcome."""
     r = mlp["router"]
     E, I, top = r["experts"], r.get("identity", 0), r["top"]
     s = softmax(w[pre + "router"] @ h)
     choice = s + w[pre + "correction"]
-    picked = sorted(range(E + I), key=lambda e: (-choice[e], e))[:top]
+    order = sorted(range(E + I), key=lambda e: (-choice[e], e))
+    picked = order[:top]
+    if margin is not None and top < E + I:
+        margin[0] = min(margin[0], choice[order[top - 1]] - choice[order[top]])
     out = np.zeros_like(h)
     for e in picked:
         out += s[e] * (h if e >= E else gated_expert(h, w, f"{pre}e{e}."))
@@ -119,15 +124,17 @@ def routed_ff(h, mlp, w, pre):
     return out
 
 
-def feed_forward(h, mlp, w, pre):
+def feed_forward(h, mlp, w, pre, margin=None):
     if mlp["kind"] == "dense":
         return w[pre + "down"] @ gelu_tanh(w[pre + "up"] @ h)
-    return routed_ff(h, mlp, w, pre)
+    return routed_ff(h, mlp, w, pre, margin)
 
 
-def forward(tokens, cfg, w, trace=None):
-    """Logits [T, V] of one sequence; ``trace`` (a list) receives x after every layer."""
+def forward(tokens, cfg, w, trace=None, margins=None):
+    """Logits [T, V] of one sequence; ``trace`` (a list) receives x after every layer,
+    ``margins`` (a list) one number per position: its closest routing decision."""
     eps = cfg["norm"]["eps"]
+    marg = [[math.inf] for _ in tokens]
     x = embed(tokens, cfg, w)
     kvs = {}
     for i, L in enumerate(cfg["layers"]):
@@ -141,9 +148,11 @@ def forward(tokens, cfg, w, trace=None):
         x = x + block_attention(us, mx, w, pre, eps, kvs[src])
         if L.get("mlp"):
             x = x + np.stack([feed_forward(scalar_norm(r, w[f"l{i}.norm2"], eps), L["mlp"], w,
-                                           f"l{i}.mlp.") for r in x])
+                                           f"l{i}.mlp.", marg[t]) for t, r in enumerate(x)])
         if trace is not None:
             trace.append(x.copy())
+    if margins is not None:
+        margins.extend(m[0] for m in marg)
     hs = np.stack([scalar_norm(r, w["final.norm"], eps) for r in x])
     return hs @ w["head"].T * cfg.get("logit_scale", 1.0)
 

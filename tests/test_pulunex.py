@@ -69,12 +69,37 @@ def tol(dtype):
     return 2e-4 if dtype == torch.float32 else 6e-2
 
 
+class Ref:
+    """Oracle logits of a sequence with each position's closest routing decision."""
+
+    def __init__(self, logits, margins):
+        self.logits, self.margins = logits, np.asarray(margins)
+
+    def __getitem__(self, k):
+        return Ref(self.logits[k], self.margins[k])
+
+
+def ref(tokens, c, w):
+    m = []
+    return Ref(O.forward(tokens, c, w, margins=m), m)
+
+
 def close(got, want, dtype, what=""):
-    """Row error as a logit comparison sees it: mean removed, relative to the spread."""
+    """Row error as a logit comparison sees it: mean removed, relative to the spread. In bf16
+    a position whose routing was a close call (the rounded input may choose another expert)
+    is held to a looser bound; every other position, and fp32 everywhere, to the strict one."""
+    loose = None
+    if isinstance(want, Ref):
+        if dtype == torch.bfloat16:
+            loose = want.margins < 0.02
+        want = want.logits
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     d = got - want
     d = d - d.mean(-1, keepdims=True)
     err = np.sqrt((d ** 2).mean(-1)) / want.std()
+    if loose is not None and loose.any():
+        assert loose.mean() < 0.2 and err[loose].max() < 8 * tol(dtype), what
+        err = err[~loose]
     assert err.max() < tol(dtype), f"{what}: error {err.max():.3g} at row {int(err.argmax())}"
 
 
@@ -213,7 +238,7 @@ def test_one_layer_models(lay, device, dtype):
     c = config([lay])
     w = O.random_weights(c, seed=3)
     t = toks(21, c["vocab"])
-    close(replay(engine(c, w, device, dtype), t, [21]), O.forward(t, c, w), dtype)
+    close(replay(engine(c, w, device, dtype), t, [21]), ref(t, c, w), dtype)
 
 
 # ------------------------------------------------------------------ schedules
@@ -221,7 +246,7 @@ def test_one_layer_models(lay, device, dtype):
 def test_prefill_equals_decode_equals_portions(device, dtype):
     w = O.random_weights(FULL, seed=5)
     t = toks(45, FULL["vocab"], 2)
-    want = O.forward(t, FULL, w)
+    want = ref(t, FULL, w)
     eng = engine(FULL, w, device, dtype)
     close(replay(eng, t, [45]), want, dtype, "whole")
     close(replay(eng, t, [1] * 45), want, dtype, "token by token")
@@ -237,7 +262,7 @@ def test_mixed_batches_and_reuse_of_pages_and_slots(device, dtype):
     state slots over time, a pool too small for all of them at once."""
     w = O.random_weights(FULL, seed=6)
     seqs = {f"r{i}": toks(n, FULL["vocab"], 10 + i) for i, n in enumerate((37, 5, 22, 1, 30, 18, 9))}
-    want = {k: O.forward(v, FULL, w) for k, v in seqs.items()}
+    want = {k: ref(v, FULL, w) for k, v in seqs.items()}
     eng = engine(FULL, w, device, dtype, max_tokens=128, live=3)
     got = {k: [] for k in seqs}
     at = {k: 0 for k in seqs}
@@ -289,7 +314,7 @@ def test_other_sizes_and_degenerate_values(device, dtype):
         w = O.random_weights(c, seed=20 + i)
         t = toks(19, c["vocab"], i)
         eng = engine(c, w, device, dtype)
-        want = O.forward(t, c, w)
+        want = ref(t, c, w)
         close(replay(eng, t, [19]), want, dtype, f"variant {i} whole")
         close(replay(eng, t, [4, 1, 1, 6, 2, 5]), want, dtype, f"variant {i} portions")
 
@@ -348,7 +373,7 @@ def test_first_tokens_and_long_decode(device, dtype):
     c = config([layer(size=5, mlp=moe()), layer(size=16, kv_from=0, mlp=dense())])
     w = O.random_weights(c, seed=12)
     t = toks(70, c["vocab"], 4)
-    want = O.forward(t, c, w)
+    want = ref(t, c, w)
     eng = engine(c, w, device, dtype)
     close(replay(eng, t, [1, 1, 2, 1] + [1] * 65), want, dtype, "from the first token on")
     close(replay(eng, t[:3], [3]), want[:3], dtype, "three tokens")
@@ -426,7 +451,64 @@ def test_model_on_matrix_core_sized_heads(gpu):
                width=64, vocab=96)
     w = O.random_weights(c, seed=31)
     t = toks(75, c["vocab"], 8)
-    want = O.forward(t, c, w)
+    want = ref(t, c, w)
     eng = engine(c, w, "cuda", torch.bfloat16, block_size=16)
     close(replay(eng, t, [75]), want, torch.bfloat16, "whole")
     close(replay(eng, t, [33, 2, 17] + [1] * 23), want, torch.bfloat16, "portions + decode")
+
+
+def _paged_case(lens, starts, H, Gk, G, dq, dv, block, seed):
+    """Random queries of portions [start, start + len) per sequence over shuffled pages; key
+    rows hold Gk heads of dq, value rows G heads of dv."""
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    nblk = [-(-(s + n) // block) for s, n in zip(starts, lens)]
+    total = sum(nblk) + 3
+    perm = torch.randperm(total, generator=g).tolist()
+    tables = torch.zeros(S, max(nblk), dtype=torch.int32)
+    at = 0
+    for s in range(S):
+        tables[s, :nblk[s]] = torch.tensor(perm[at:at + nblk[s]], dtype=torch.int32)
+        at += nblk[s]
+    kc = torch.randn(total * block, Gk * dq, generator=g).to(torch.bfloat16)
+    vc = torch.randn(total * block, G * dv, generator=g).to(torch.bfloat16)
+    q = torch.randn(sum(lens), H * dq, generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    pos = torch.cat([torch.arange(s, s + n, dtype=torch.int32) for s, n in zip(starts, lens)])
+    return q, kc, vc, cu, pos, tables
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H_,G,dq,dv,size", [(4, 2, 64, 48, 40), (6, 2, 128, 64, 96),
+                                             (16, 4, 256, 128, 19), (3, 1, 32, 16, 1),
+                                             (8, 8, 512, 32, 1000), (12, 3, 96, 80, 33)])
+@pytest.mark.parametrize("decode", [False, True])
+def test_matrix_core_attention_with_blocks_and_shared_key_rows(gpu, H_, G, dq, dv, size, decode):
+    """The MFMA form with the block mask and one key head per cache row against the PyTorch
+    reference: prompt portions whose query tiles straddle block edges, and decode rows with long
+    contexts (key splits), at block edges, one after an edge, and at position 0."""
+    from distributed_llm_inferencing_amd.ops import reference as R
+    if decode:
+        starts = [size - 1, size, 2 * size + size // 2, 0, 777, 5 * size - 1]
+        lens = [1] * len(starts)
+    else:
+        lens, starts = [37, 1, 16, 50, 2], [0, 63, 48, 200, size]
+    block = 16
+    q, kc, vc, cu, pos, bt = _paged_case(lens, starts, H_, 1, G, dq, dv, block, seed=H_ + dq)
+    scale = 1.0 / dq ** 0.5
+    want = R.window_attention(q, kc, vc, dq, dv, H_, G, cu, pos, bt, block, 1 << 30, scale,
+                              out_dtype=torch.float32, chunk=size, k_groups=1)
+    d = lambda t: t.to(gpu)      # noqa: E731
+    args = (d(q), d(kc), d(vc), dq, dv, H_, G, d(cu), max(lens), d(pos), d(bt), block, 1 << 30,
+            scale)
+    assert H.MFMA_ATTENTION
+    got = H.window_attention(*args, chunk=size, k_groups=1).float().cpu()
+    H.MFMA_ATTENTION = False
+    try:
+        scalar = H.window_attention(*args, chunk=size, k_groups=1).float().cpu()
+    finally:
+        H.MFMA_ATTENTION = True
+    lim = 0.03 * want.abs().max().item() + 0.02
+    assert (scalar - want).abs().max() < lim
+    assert (got - want).abs().max() < lim
+    assert not torch.equal(got, scalar)                   # the two kernels really differ
