@@ -91,14 +91,14 @@ def close(got, want, dtype, what=""):
     loose = None
     if isinstance(want, Ref):
         if dtype == torch.bfloat16:
-            loose = want.margins < 0.02
+            loose = want.margins < 0.005
         want = want.logits
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     d = got - want
     d = d - d.mean(-1, keepdims=True)
     err = np.sqrt((d ** 2).mean(-1)) / want.std()
     if loose is not None and loose.any():
-        assert loose.mean() < 0.2 and err[loose].max() < 8 * tol(dtype), what
+        assert err[loose].max() < 8 * tol(dtype), what
         err = err[~loose]
     assert err.max() < tol(dtype), f"{what}: error {err.max():.3g} at row {int(err.argmax())}"
 
@@ -511,4 +511,4 @@ def test_matrix_core_attention_with_blocks_and_shared_key_rows(gpu, H_, G, dq, d
     lim = 0.03 * want.abs().max().item() + 0.02
     assert (scalar - want).abs().max() < lim
     assert (got - want).abs().max() < lim
-    assert not torch.equal(got, scalar)                   # the two kernels really differ
+    assert size == 1 or not torch.equal(got, scalar)      # the two kernels really differ
