@@ -67,6 +67,92 @@ def _like_for_like_value():
         return None
 
 
+def run_design_pulunex(a):
+    """``--design pulunex``: prefill and decode throughput of the design at layer sizes of a
+    real model (random weights) beside the framework's closest model, a Mixtral of equal width,
+    depth, heads, experts, expert width and experts per token, both through ``LLMEngine``."""
+    from dataclasses import replace
+    from distributed_llm_inferencing_amd.engine import SamplingParams
+    from distributed_llm_inferencing_amd.engine.llm_engine import LLMEngine
+    from distributed_llm_inferencing_amd.models.configs import LayerSpec, get_config, hybrid_config
+    D, Fw, V, Hh, G, hd = a.design_width, a.design_ff, 32000, a.design_width // 128, 8, 128
+    E, top, chunk = 8, 2, a.design_window
+
+    def lay(kv_from=-1):
+        return LayerSpec("talk_attention", heads=Hh, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5,
+                         chunk=chunk, kv_from=kv_from, shift=True, ff_kind="moe", ff=Fw,
+                         experts=E, identity=2, top=top, shared_ff=2048)
+    hyb = hybrid_config("pulunex-bench", D, V, (lay(), lay(), lay(1), lay(1)), arch="pulunex",
+                        max_position=1 << 15, embed_scale=8.0, logit_scale=0.5, learned_pos=True,
+                        scalar_norm=True)
+    mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
+                  num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,
+                  num_experts=E, top_k_experts=top, max_position=1 << 15)
+    rng = np.random.default_rng(0)
+    out = {}
+    for cfg in (hyb, mix):
+        if cfg.name.split("-")[0] not in a.design_models.split(","):
+            continue
+        res = {}
+        for (S, L) in a.design_prefill:
+            eng = LLMEngine(cfg, device="cuda:0", max_batch=max(S, 8), max_model_len=L + 64,
+                            block_size=16, max_kv_tokens=S * (L + 64) + 4096,
+                            max_prefill_tokens=S * L, use_graphs=False, lookahead=False)
+            prompts = [rng.integers(0, V, L).tolist() for _ in range(S)]
+            sp = SamplingParams(max_new_tokens=1, ignore_eos=True)
+            ts = []
+            for _ in range(a.warmup + a.steps):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                eng.generate(prompts, sp)
+                torch.cuda.synchronize()
+                ts.append(time.perf_counter() - t0)
+            res[f"prefill_{S}x{L}_tok_s"] = round(S * L / min(ts[a.warmup:]), 1)
+            del eng
+            torch.cuda.empty_cache()
+        for (B, C) in a.design_decode:
+            n_new = 33
+            eng = LLMEngine(cfg, device="cuda:0", max_batch=B, max_model_len=C + n_new + 16,
+                            block_size=16, max_kv_tokens=B * (C + n_new + 32) + 4096,
+                            max_prefill_tokens=max(8192, C))
+            eng.warmup(buckets=[B])
+            prompts = [rng.integers(0, V, C).tolist() for _ in range(B)]
+
+            def decode_steps(n):
+                """Admit the batch, run its prefill, then time n pure decode steps."""
+                sp = SamplingParams(max_new_tokens=n + 8, ignore_eos=True)
+                for p in prompts:
+                    eng.add_request(p, sp)
+                sch = eng.scheduler
+                while sch.waiting or any(sch.prefilling):
+                    eng.step()
+                for _ in range(3):
+                    eng.step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    eng.step()
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / n
+                while eng.has_work():
+                    eng.step()
+                return dt
+            decode_steps(4)
+            best = min(decode_steps(n_new - 1) for _ in range(max(1, a.steps)))
+            res[f"decode_b{B}_ctx{C}_tok_s"] = round(B / best, 1)
+            res[f"decode_b{B}_ctx{C}_ms_per_step"] = round(1000 * best, 3)
+            del eng
+            torch.cuda.empty_cache()
+        out[cfg.name] = res
+    print(json.dumps({"metric": "prefill and decode tokens/s, Pulunex design vs Mixtral of equal "
+                                "size (random weights)", "unit": "tokens/s", "n_gpus": 1,
+                      "dtype": "bf16", "data": "synthetic prompts, random-init weights",
+                      "config": {"width": D, "expert_ff": Fw, "layers": 4, "heads": Hh,
+                                 "kv_heads": G, "head_dim": hd, "block": chunk, "experts": E,
+                                 "identity_experts": 2, "top": top, "shared_ff": 2048},
+                      "results": out}), flush=True)
+
+
 def run_design(a):
     """``--design buborax``: prefill and decode throughput of the hybrid design at layer sizes
     of a real model (random weights), beside a Llama of equal width, depth (= layer runs),
@@ -291,10 +377,12 @@ def main():
                     help="N>1: pp = layer-sharded pipeline (dense, default), ep = expert "
                          "parallel (MoE), tp = tensor-parallel ablation, dp = independent "
                          "replicas")
-    ap.add_argument("--design", default=None, choices=["buborax"],
+    ap.add_argument("--design", default=None, choices=["buborax", "pulunex"],
                     help="instead of the headline workload: prefill / decode throughput of "
-                         "this design at real layer sizes beside a Llama of equal size")
-    ap.add_argument("--design-models", default="buborax,llama", help="which of the two to run")
+                         "this design at real layer sizes beside the closest model of equal "
+                         "size (buborax: Llama, pulunex: Mixtral)")
+    ap.add_argument("--design-models", default="buborax,llama,pulunex,mixtral",
+                    help="which of the design and its comparison model to run")
     ap.add_argument("--design-width", type=int, default=4096)
     ap.add_argument("--design-ff", type=int, default=14336)
     ap.add_argument("--design-window", type=int, default=1024)
@@ -305,7 +393,7 @@ def main():
     a = ap.parse_args()
     if a.design:
         _heartbeat()
-        return run_design(a)
+        return run_design_pulunex(a) if a.design == "pulunex" else run_design(a)
 
     from distributed_llm_inferencing_amd import launch
     if a.gpus > 1 and not launch.under_launcher():

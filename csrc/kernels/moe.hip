@@ -470,19 +470,22 @@ __global__ void __launch_bounds__(256) score_router_kernel(
 }
 
 // out[t] = sum_j w[t][j] * (routed ? y[pos[t][j]] : identity ? x[t] : 0) + gate[t] * ys[t]
-// y, ys fp32; x storage type; ids >= n_real are identity experts (their pos is -1).
+// y, ys fp32; x storage type; ids >= n_real are identity experts (their pos is -1). With
+// `routed` (storage type [T, dim]: the real experts' weighted sum, already combined) instead
+// of y / pos, only the identity and shared parts are added to it.
 template <typename S>
 __global__ void __launch_bounds__(256) moe_combine_f32_kernel(
-    float* __restrict__ out, const float* __restrict__ y, const float* __restrict__ w,
+    float* __restrict__ out, const float* __restrict__ y, const S* __restrict__ routed,
+    const float* __restrict__ w,
     const int* __restrict__ pos, const int* __restrict__ ids, const S* __restrict__ x, int ldx,
     const float* __restrict__ ys, const float* __restrict__ gate, int ldg, int T, int k, int dim,
     int n_real) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= (long)T * dim) return;
   const int t = (int)(gid / dim), c = (int)(gid % dim);
-  float acc = 0.f;
+  float acc = routed != nullptr ? rld(routed + gid) : 0.f;
   for (int j = 0; j < k; ++j) {
-    const int p = pos[t * k + j];
+    const int p = pos != nullptr ? pos[t * k + j] : -1;
     const float ww = w[t * k + j];
     if (p >= 0) acc += ww * y[(long)p * dim + c];
     else if (ids[t * k + j] >= n_real) acc += ww * rld(x + (long)t * ldx + c);
@@ -511,19 +514,23 @@ extern "C" int dli_score_router(float* topk_w, int* topk_ids, float* gates, cons
   DLI_RETURN_LAUNCH();
 }
 
-extern "C" int dli_moe_combine_f32(float* out, const float* y, const float* w, const int* pos,
-                                   const int* ids, const void* x, int ldx, const float* ys,
-                                   const float* gate, int ldg, int T, int k, int dim, int n_real,
-                                   int dt, hipStream_t st) {
+extern "C" int dli_moe_combine_f32(float* out, const float* y, const void* routed,
+                                   const float* w, const int* pos, const int* ids, const void* x,
+                                   int ldx, const float* ys, const float* gate, int ldg, int T,
+                                   int k, int dim, int n_real, int dt, hipStream_t st) {
   if (T <= 0) return 0;
-  if ((ys == nullptr) != (gate == nullptr)) return (int)hipErrorInvalidValue;
+  if ((ys == nullptr) != (gate == nullptr) || (y == nullptr) != (pos == nullptr) ||
+      (y == nullptr) == (routed == nullptr))
+    return (int)hipErrorInvalidValue;
   const int nb = (int)(((long)T * dim + 255) / 256);
   if (dt == 0)
-    moe_combine_f32_kernel<u16><<<nb, 256, 0, st>>>(out, y, w, pos, ids, (const u16*)x, ldx, ys,
-                                                    gate, ldg, T, k, dim, n_real);
+    moe_combine_f32_kernel<u16><<<nb, 256, 0, st>>>(out, y, (const u16*)routed, w, pos, ids,
+                                                    (const u16*)x, ldx, ys, gate, ldg, T, k, dim,
+                                                    n_real);
   else if (dt == 1)
-    moe_combine_f32_kernel<float><<<nb, 256, 0, st>>>(out, y, w, pos, ids, (const float*)x, ldx,
-                                                      ys, gate, ldg, T, k, dim, n_real);
+    moe_combine_f32_kernel<float><<<nb, 256, 0, st>>>(out, y, (const float*)routed, w, pos, ids,
+                                                      (const float*)x, ldx, ys, gate, ldg, T, k,
+                                                      dim, n_real);
   else return (int)hipErrorInvalidValue;
   DLI_RETURN_LAUNCH();
 }

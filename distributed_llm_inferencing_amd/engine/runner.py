@@ -260,6 +260,8 @@ class StageRunner:
                 normed = {(lp["wqkv"].shape[0], lp["wqkv"].shape[1], "splitk"),
                           (lp["w_gu"].shape[0], lp["w_gu"].shape[1], "silu_mul")}
             G.autotune(shapes, weights, self.device, log=log, qkv_heads=qkv, normed_in=normed)
+            for rows, w, epi in getattr(m, "grouped_gemm_shapes", lambda _b: [])(b):
+                G.autotune_grouped(rows, w, epi, log=log)
             if moe:      # grouped expert GEMMs: rows = b tokens x top-k (uniform routing)
                 lp = m.layers[0]
                 rows = b * m.cfg.top_k_experts

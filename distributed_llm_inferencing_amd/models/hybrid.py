@@ -26,7 +26,8 @@ import torch
 from ..engine.batch import DeviceBatch
 from ..ops import hybrid as H
 from .configs import ModelConfig
-from .mixers import FEED_FORWARDS, MIXERS, StepView, derive_constants
+from .mixers import (FEED_FORWARDS, MIXERS, StepView, derive_constants,
+                     prepare_feed_forward)
 from .model import TransformerLM
 
 
@@ -39,6 +40,8 @@ class HybridLM(TransformerLM):
         if layer_start != 0 or (layer_end is not None and layer_end != cfg.num_layers):
             raise ValueError("hybrid designs run on one stage (the loop entry reads the "
                              "embedding output)")
+        for i, spec in enumerate(cfg.layer_specs):
+            prepare_feed_forward(spec, params, f"layers.{i}.")
         super().__init__(cfg, params, 0, None, device)
         self.dtype = params["embed"].dtype
         self.runs = cfg.layer_runs()
@@ -50,6 +53,9 @@ class HybridLM(TransformerLM):
 
     def to(self, device):
         super().to(device)
+        for i, spec in enumerate(self.cfg.layer_specs):
+            prepare_feed_forward(spec, self.params, f"layers.{i}.")
+        self.layers = [self._layer_params(i) for i in range(len(self.cfg.layer_specs))]
         for spec, lp in zip(self.cfg.layer_specs, self.layers):
             derive_constants(spec, lp, self.device)
         self._cu.clear()
@@ -150,9 +156,31 @@ class HybridLM(TransformerLM):
         mats = [w for lp in self.layers for w in lp.values()
                 if isinstance(w, torch.Tensor) and w.dim() == 2 and w.dtype == self.dtype]
         mats += [self.params[k] for k in ("loop_in", "lm_head") if k in self.params]
+        fused = {}                     # first GEMMs of feed-forwards in the tuned layout
+        for spec, lp in zip(self.cfg.layer_specs, self.layers):
+            if "ff_tuned" in lp:
+                if spec.ff_kind == "gelu":
+                    fused[id(lp["w_up"])] = "bias_gelu"
+                elif spec.shared_ff:
+                    fused[id(lp["ws_gu"])] = "silu_mul"
         for w in mats:
             n, k = w.shape
-            if k % 64 == 0 and (n, k) not in weights and n >= 16:
-                shapes.append((M, n, k, "f32"))
-                weights[(n, k)] = w
-        return shapes, weights
+            epi = fused.get(id(w), "f32")
+            if k % 64 == 0 and (n, k, epi) not in weights and n >= 16:
+                shapes.append((M, n, k, epi))
+                weights[(n, k, epi)] = w
+        # the autotune keys weights by (n, k)
+        return shapes, {(n, k): w for (n, k, _), w in weights.items()}
+
+    def grouped_gemm_shapes(self, M: int):
+        """(rows, expert weights, epilogue) of the grouped expert GEMMs a step of M rows runs
+        on the tuned tile family (uniform routing: M x top rows over the experts)."""
+        out, seen = [], set()
+        for spec, lp in zip(self.cfg.layer_specs, self.layers):
+            if spec.ff_kind == "moe" and "ff_tuned" in lp:
+                key = (tuple(lp["w_gu"].shape), spec.top)
+                if key not in seen:
+                    seen.add(key)
+                    rows = M * spec.top
+                    out += [(rows, lp["w_gu"], "silu_mul"), (rows, lp["w_down"], "none")]
+        return out

@@ -120,13 +120,44 @@ MIXERS = {"attention": attention_mixer, "hgrn2": hgrn2_mixer,
 
 
 # ----------------------------------------------------------------------------- feed-forwards
+# Two layouts of a feed-forward's weights. The plain one ([gate | up] stacked) runs the
+# shape-agnostic GEMM with fp32 outputs and separate activation kernels: any sizes, bf16 or
+# fp32. The tuned one (``prepare_feed_forward``: bf16, sizes the tile family takes) fuses the
+# activation into the first GEMM's epilogue — SiLU * up over the 16-row interleaved gate/up
+# weight, bias + GELU for the ungated form — and runs the experts as the grouped GEMMs of the
+# framework's other mixture model.
+def prepare_feed_forward(spec: LayerSpec, params: dict, pre: str) -> None:
+    """Re-lay the feed-forward weights of layer ``pre`` for the tuned GEMMs when they fit
+    (in ``params``, in place; marked by ``<pre>ff_tuned`` so that it happens once)."""
+    from ..ops.reference import interleave_gate_up
+    w = params.get(pre + "w_down")
+    if (not spec.ff or w is None or pre + "ff_tuned" in params or w.dtype != torch.bfloat16
+            or not w.is_cuda or spec.ff_kind not in ("gelu", "moe") or w.shape[-2] % 64
+            or spec.ff % 64 or spec.shared_ff % 64):
+        return
+    if spec.ff_kind == "gelu":
+        params[pre + "b_up"] = torch.zeros(spec.ff, dtype=w.dtype, device=w.device)
+    else:
+        gu = params[pre + "w_gu"]
+        for e in range(gu.shape[0]):                 # expert by expert: no second full copy
+            gu[e] = interleave_gate_up(gu[e, :spec.ff].clone(), gu[e, spec.ff:].clone())
+        if spec.shared_ff:
+            s = params[pre + "ws_gu"]
+            params[pre + "ws_gu"] = interleave_gate_up(s[:spec.shared_ff], s[spec.shared_ff:]).contiguous()
+    params[pre + "ff_tuned"] = torch.ones(1, dtype=torch.int8, device=w.device)
+
+
 def gated_gelu_ff(spec: LayerSpec, lp: dict, h):
     act = H.act_mul(H.linear_any(h, lp["w_gu"]), spec.ff, h.dtype, "gelu_mul")
     return H.linear_any(act, lp["w_down"])
 
 
 def gelu_ff(spec: LayerSpec, lp: dict, h):
-    act = H.act_mul(H.linear_any(h, lp["w_up"]), spec.ff, h.dtype, "gelu")
+    if "ff_tuned" in lp:
+        from .. import ops
+        act = ops.linear(h, lp["w_up"], lp["b_up"], epi="bias_gelu")
+    else:
+        act = H.act_mul(H.linear_any(h, lp["w_up"]), spec.ff, h.dtype, "gelu")
     return H.linear_any(act, lp["w_down"])
 
 
@@ -134,8 +165,16 @@ def moe_ff(spec: LayerSpec, lp: dict, h):
     """Routed gated-SiLU experts + identity experts + a gated shared expert, summed in fp32."""
     ng = 1 if spec.shared_ff else 0
     tw, ti, gates = H.score_router(h, lp["router"], lp["correction"], spec.top, ng)
-    shared = (lp["ws_gu"], lp["ws_down"], gates) if ng else None
-    return H.moe_experts_f32(h, lp["w_gu"], lp["w_down"], tw, ti, shared)
+    if "ff_tuned" not in lp:
+        shared = (lp["ws_gu"], lp["ws_down"], gates) if ng else None
+        return H.moe_experts_f32(h, lp["w_gu"], lp["w_down"], tw, ti, shared)
+    from .. import ops
+    # ids from E on (identity experts) match no local expert and add nothing here
+    routed = ops.moe_mlp(h, lp["w_gu"], lp["w_down"], tw, ti, 0)
+    ys = None
+    if ng:
+        ys = H.linear_any(ops.linear(h, lp["ws_gu"], epi="silu_mul"), lp["ws_down"])
+    return H.moe_finish(routed, tw, ti, h, lp["w_gu"].shape[0], ys, gates if ng else None)
 
 
 FEED_FORWARDS = {"gated_gelu": gated_gelu_ff, "gelu": gelu_ff, "moe": moe_ff}

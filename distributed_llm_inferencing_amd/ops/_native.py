@@ -80,7 +80,7 @@ _SIGS = {
     "dli_talk_prepare": [P, I, P, P, F, I, I, I, I, I, P, P, P, P, I, P],
     "dli_score_router": [P, P, P, P, I, P, P, I, I, I, I, I, I, P],
     "dli_gemm_any_grouped": [P, L, P, L, L, P, L, I, I, I, I, I, P, P, P],
-    "dli_moe_combine_f32": [P, P, P, P, P, P, I, P, P, I, I, I, I, I, I, P],
+    "dli_moe_combine_f32": [P, P, P, P, P, P, P, I, P, P, I, I, I, I, I, I, P],
     "dli_concat_cast": [P, P, P, I, I, I, P],
     "dli_attn_prepare": [P, I, P, P, F, I, I, I, I, P, P, P, P, I, P],
     "dli_mla_prepare": [P, I, P, F, I, I, I, I, I, I, P, P, P, P, P, P, I, P],

@@ -359,7 +359,23 @@ def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None) -> torch.Ten
         a = act_mul(linear_any(x, ws_gu), ws_gu.shape[0] // 2, x.dtype, "silu_mul")
         ys = linear_any(a, ws_down)
     out = torch.empty(T, D, dtype=torch.float32, device=dev)
-    _call("dli_moe_combine_f32", _p(out), _p(y), _p(topk_w), _p(pos), _p(topk_ids), _p(x), x.stride(0),
-          _p(ys), _p(gate), gate.stride(0) if gate is not None else 0, T, k, D, E,
+    _call("dli_moe_combine_f32", _p(out), _p(y), None, _p(topk_w), _p(pos), _p(topk_ids), _p(x),
+          x.stride(0), _p(ys), _p(gate), gate.stride(0) if gate is not None else 0, T, k, D, E,
           _dt(x.dtype), _st())
+    return out
+
+
+def moe_finish(routed, topk_w, topk_ids, x, n_real: int, ys=None, gate=None) -> torch.Tensor:
+    """fp32 [T, D]: ``routed`` (the weighted sum of the real experts, storage dtype) + the
+    identity experts' share (weights of ids >= n_real) * x + gate * ys (the shared expert)."""
+    T, D = x.shape
+    if not x.is_cuda:
+        out = routed.float() + (topk_w * (topk_ids >= n_real)).sum(-1, keepdim=True) * x.float()
+        if ys is not None:
+            out = out + gate.float().reshape(T, 1) * ys.float()
+        return out
+    out = torch.empty(T, D, dtype=torch.float32, device=x.device)
+    _call("dli_moe_combine_f32", _p(out), None, _p(routed), _p(topk_w), None, _p(topk_ids),
+          _p(x), x.stride(0), _p(ys), _p(gate), gate.stride(0) if gate is not None else 0, T,
+          topk_ids.shape[1], D, n_real, _dt(x.dtype), _st())
     return out

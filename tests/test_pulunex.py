@@ -444,15 +444,18 @@ def test_registry_model_random_init_generates():
 
 @pytest.mark.gpu
 def test_model_on_matrix_core_sized_heads(gpu):
-    """Head sizes the MFMA attention takes (multiples of 32 / 16), prompts long enough for
-    several query tiles, blocks that end inside a tile."""
-    c = config([layer(heads=4, kv=2, dim=32, vdim=48, size=40, mlp=moe(ff=32, shared=64)),
-                layer(heads=4, kv=2, dim=32, vdim=48, size=19, kv_from=0, mlp=dense(64))],
+    """Head sizes the MFMA attention takes (multiples of 32 / 16) and feed-forward sizes the
+    tuned GEMM tiles take (fused activation epilogues, grouped expert GEMMs); prompts long
+    enough for several query tiles, blocks that end inside a tile."""
+    c = config([layer(heads=4, kv=2, dim=32, vdim=48, size=40, mlp=moe(ff=64, shared=128)),
+                layer(heads=4, kv=2, dim=32, vdim=48, size=19, kv_from=0, mlp=dense(64)),
+                layer(heads=4, kv=2, dim=32, vdim=48, size=64, mlp=moe(ff=64, identity=0, shared=0))],
                width=64, vocab=96)
     w = O.random_weights(c, seed=31)
     t = toks(75, c["vocab"], 8)
     want = ref(t, c, w)
     eng = engine(c, w, "cuda", torch.bfloat16, block_size=16)
+    assert all("ff_tuned" in lp for lp in eng.model.layers)
     close(replay(eng, t, [75]), want, torch.bfloat16, "whole")
     close(replay(eng, t, [33, 2, 17] + [1] * 23), want, torch.bfloat16, "portions + decode")
 
