@@ -119,13 +119,14 @@ __global__ void __launch_bounds__(256) resadd_groupnorm_kernel(
 }
 
 // Token shift over normed fp32 rows: u[t] = h[t] + (h[t-1] - h[t]) * mu. Grid (row blocks of a
-// sequence, sequences). h[t-1] of a portion's first row is the sequence's row of `state`
-// (zeros at position 0). The workgroup that holds a portion's first row also stores the
-// portion's LAST row into the state, after it has read the old one: every thread reads and
+// sequence, sequences, column blocks). h[t-1] of a portion's first row is the sequence's row
+// of `state` (zeros at position 0). The workgroup that holds a portion's first row also stores
+// the portion's LAST row into the state, after it has read the old one: every thread reads and
 // then writes the same columns, so the order holds without a second launch. Sequences
-// without a slot (padding rows of a captured step) pass through unshifted.
+// without a slot (padding rows of a captured step) pass through unshifted. VEC = 4: 16-byte
+// loads of the fp32 rows (dim a multiple of 4).
 constexpr int SHIFT_ROWS = 4;
-template <typename S>
+template <typename S, int VEC>
 __global__ void __launch_bounds__(256) token_shift_kernel(
     const float* __restrict__ h, const S* __restrict__ mu, float* __restrict__ state,
     const int* __restrict__ slots, const int* __restrict__ cu, const int* __restrict__ positions,
@@ -137,18 +138,34 @@ __global__ void __launch_bounds__(256) token_shift_kernel(
   const int slot = slots != nullptr ? slots[s] : -1;
   const int rows = min(SHIFT_ROWS, t1 - t0 - r0);
   const bool from_zero = positions[t0] == 0;
-  for (int c = threadIdx.x; c < dim; c += blockDim.x) {
-    const float m = ldf(mu + c);
-    float prev;
-    if (r0 > 0) prev = h[(long)(t0 + r0 - 1) * dim + c];
-    else prev = (slot < 0 || from_zero) ? 0.f : state[(long)slot * dim + c];
-    for (int i = 0; i < rows; ++i) {
-      const long o = (long)(t0 + r0 + i) * dim + c;
-      const float cur = h[o];
-      stf(out + o, slot < 0 ? cur : cur + (prev - cur) * m);
-      prev = cur;
+  const int c = (blockIdx.z * blockDim.x + threadIdx.x) * VEC;
+  if (c >= dim) return;
+  float m[VEC], prev[VEC], cur[VEC];
+#pragma unroll
+  for (int u = 0; u < VEC; ++u) { m[u] = ldf(mu + c + u); prev[u] = 0.f; }
+  auto load = [&](const float* p, float* v) {
+    if constexpr (VEC == 4) {
+      const f32x4 q = *reinterpret_cast<const f32x4*>(p);
+      v[0] = q[0]; v[1] = q[1]; v[2] = q[2]; v[3] = q[3];
+    } else {
+      v[0] = *p;
     }
-    if (r0 == 0 && slot >= 0) state[(long)slot * dim + c] = h[(long)(t1 - 1) * dim + c];
+  };
+  if (r0 > 0) load(h + (long)(t0 + r0 - 1) * dim + c, prev);
+  else if (slot >= 0 && !from_zero) load(state + (long)slot * dim + c, prev);
+  for (int i = 0; i < rows; ++i) {
+    const long o = (long)(t0 + r0 + i) * dim + c;
+    load(h + o, cur);
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) {
+      stf(out + o + u, slot < 0 ? cur[u] : cur[u] + (prev[u] - cur[u]) * m[u]);
+      prev[u] = cur[u];
+    }
+  }
+  if (r0 == 0 && slot >= 0) {
+    load(h + (long)(t1 - 1) * dim + c, cur);
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) state[(long)slot * dim + c + u] = cur[u];
   }
 }
 
@@ -204,24 +221,28 @@ __global__ void __launch_bounds__(256) act_mul4_kernel(
   for (int i = 0; i < 4; ++i) stf(out + (long)t * ldo + c + i, act_pair(kind, g[i], u[i]));
 }
 
-// One workgroup per token. proj row (fp32, + bias): [H*d q | G*d k | G*dv v] (q only when the
+// Grid (token, head slices). proj row (fp32, + bias): [H*d q | G*d k | G*dv v] (q only when the
 // layer attends another layer's cache: kcache null). q and k heads are divided by their RMS;
-// k and v go to the cache row; the queries leave with the pre-softmax head mixing folded in:
+// k and v go to the cache row (by slice 0); the queries leave with the pre-softmax head mixing
+// folded in:
 //   sum_g talk[h][g] (q_g . k_c(g)) = sum_c (sum_{g in c} talk[h][g] q_g) . k_c
 // so head h carries q'_h [G*d] whose part c is sum_{g in c} talk[h][g] q_g, and scores whole
-// cached key rows.
-template <typename S>
+// cached key rows. Every slice norms all query heads (cheap) and writes the mixed queries of
+// its own heads [h0, h1), VEC consecutive columns a thread.
+template <typename S, int VEC>
 __global__ void __launch_bounds__(256) talk_prepare_kernel(
     const float* __restrict__ proj, int ldp, const S* __restrict__ bias,
     const float* __restrict__ talk, float eps, int H, int G, int d, int dv,
     S* __restrict__ q_out, S* __restrict__ kcache, S* __restrict__ vcache,
     const int* __restrict__ slots) {
-  extern __shared__ float qn[];                       // [H * d] unit-RMS queries
+  extern __shared__ __attribute__((aligned(16))) float qn[];   // [H * d] unit-RMS queries, [H * H] talk
+  float* tk = qn + H * d;
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const float* row = proj + (long)t * ldp;
-  const int slot = kcache != nullptr ? slots[t] : -1;
+  const int slot = (kcache != nullptr && blockIdx.y == 0) ? slots[t] : -1;
   const int units = H + (slot >= 0 ? G : 0);
+  for (int i = threadIdx.x; i < H * H; i += blockDim.x) tk[i] = talk[i];
   for (int u = wid; u < units; u += nw) {
     const int off = u * d;                            // q heads, then k heads, are contiguous
     float ss = 0.f;
@@ -243,14 +264,27 @@ __global__ void __launch_bounds__(256) talk_prepare_kernel(
   }
   __syncthreads();
   const int rep = H / G, wq = G * d;
+  const int per = (H + gridDim.y - 1) / gridDim.y;
+  const int h0 = blockIdx.y * per, h1 = min(H, h0 + per);
   S* qo = q_out + (long)t * H * wq;
-  for (int i = threadIdx.x; i < H * wq; i += blockDim.x) {
-    const int h = i / wq, rem = i % wq, c = rem / d, col = rem % d;
-    const float* tk = talk + h * H + c * rep;
+  for (int i = h0 * wq + threadIdx.x * VEC; i < h1 * wq; i += blockDim.x * VEC) {
+    const int h = i / wq, rem = i % wq, c = rem / d, col = rem % d;   // VEC | d: one (h, c)
+    const float* tr = tk + h * H + c * rep;
     const float* qs = qn + (c * rep) * d + col;
-    float acc = 0.f;
-    for (int r = 0; r < rep; ++r) acc += tk[r] * qs[r * d];
-    stf(qo + i, acc);
+    float acc[VEC];
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) acc[u] = 0.f;
+    for (int r = 0; r < rep; ++r) {
+      const float w = tr[r];
+#pragma unroll
+      for (int u = 0; u < VEC; ++u) acc[u] += w * qs[r * d + u];
+    }
+    if constexpr (VEC == 8 && sizeof(S) == 2) {
+      store8((u16*)qo + i, acc);
+    } else {
+#pragma unroll
+      for (int u = 0; u < VEC; ++u) stf(qo + i + u, acc[u]);
+    }
   }
 }
 
@@ -402,12 +436,15 @@ extern "C" int dli_token_shift(const float* h, const void* mu, float* state, con
                                int max_seqlen, int dim, int dt, hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
   if (num_seqs > 65535) return (int)hipErrorInvalidValue;
-  dim3 grid((max_seqlen + SHIFT_ROWS - 1) / SHIFT_ROWS, num_seqs);
-  DT_SWITCH(dt,
-            (token_shift_kernel<u16><<<grid, 256, 0, st>>>(h, (const u16*)mu, state, slots, cu,
-                                                          positions, (u16*)out, dim)),
-            (token_shift_kernel<float><<<grid, 256, 0, st>>>(h, (const float*)mu, state, slots, cu,
-                                                            positions, (float*)out, dim)));
+  const bool v4 = dim % 4 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)state % 16 == 0;
+  const int per = 256 * (v4 ? 4 : 1);
+  dim3 grid((max_seqlen + SHIFT_ROWS - 1) / SHIFT_ROWS, num_seqs, (dim + per - 1) / per);
+#define SHIFT_LAUNCH(S, V)                                                                    \
+  token_shift_kernel<S, V><<<grid, 256, 0, st>>>(h, (const S*)mu, state, slots, cu, positions, \
+                                                 (S*)out, dim)
+  if (v4) DT_SWITCH(dt, (SHIFT_LAUNCH(u16, 4)), (SHIFT_LAUNCH(float, 4)));
+  else DT_SWITCH(dt, (SHIFT_LAUNCH(u16, 1)), (SHIFT_LAUNCH(float, 1)));
+#undef SHIFT_LAUNCH
   DLI_RETURN_LAUNCH();
 }
 
@@ -435,15 +472,20 @@ extern "C" int dli_talk_prepare(const float* proj, int ldp, const void* bias, co
   if (T <= 0) return 0;
   if (H < 1 || G < 1 || H % G || d < 1 || dv < 1 || (kcache == nullptr) != (vcache == nullptr))
     return (int)hipErrorInvalidValue;
-  const size_t sh = (size_t)H * d * 4;
+  const size_t sh = ((size_t)H * d + (size_t)H * H) * 4;
   if (sh > 60000) return (int)hipErrorInvalidValue;
-  DT_SWITCH(dt,
-            (talk_prepare_kernel<u16><<<T, 256, sh, st>>>(
-                proj, ldp, (const u16*)bias, talk, eps, H, G, d, dv, (u16*)q_out, (u16*)kcache,
-                (u16*)vcache, slots)),
-            (talk_prepare_kernel<float><<<T, 256, sh, st>>>(
-                proj, ldp, (const float*)bias, talk, eps, H, G, d, dv, (float*)q_out,
-                (float*)kcache, (float*)vcache, slots)));
+  // few tokens (decode steps): the heads of a token are dealt to several workgroups
+  int slices = 1;
+  while (slices < H && slices < 16 && (long)T * slices < 1024) slices *= 2;
+  if (slices > H) slices = H;
+  dim3 grid(T, slices);
+  const bool v8 = d % 8 == 0 && (uintptr_t)q_out % 16 == 0;
+#define TALK_LAUNCH(S, V)                                                                   \
+  talk_prepare_kernel<S, V><<<grid, 256, sh, st>>>(proj, ldp, (const S*)bias, talk, eps, H, G, \
+                                                   d, dv, (S*)q_out, (S*)kcache, (S*)vcache, slots)
+  if (v8) DT_SWITCH(dt, (TALK_LAUNCH(u16, 8)), (TALK_LAUNCH(float, 8)));
+  else DT_SWITCH(dt, (TALK_LAUNCH(u16, 1)), (TALK_LAUNCH(float, 1)));
+#undef TALK_LAUNCH
   DLI_RETURN_LAUNCH();
 }
 

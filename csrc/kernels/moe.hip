@@ -430,20 +430,53 @@ template <typename S>
 __global__ void __launch_bounds__(256) score_router_kernel(
     float* __restrict__ topk_w, int* __restrict__ topk_ids, float* __restrict__ gates,
     const S* __restrict__ h, int ldh, const S* __restrict__ W, const float* __restrict__ corr,
-    int D, int n, int n_gate, int top) {
-  extern __shared__ float rsm[];                      // [D] row, [n + n_gate] logits
+    int D, int n, int n_gate, int top, bool vec) {
+  extern __shared__ __attribute__((aligned(16))) float rsm[];                      // [D] row, [n + n_gate] logits
   float* row = rsm;
   float* z = rsm + D;
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int c = threadIdx.x; c < D; c += blockDim.x) row[c] = rld(h + (long)t * ldh + c);
   __syncthreads();
-  for (int e = wid; e < n + n_gate; e += nw) {
-    const S* wr = W + (long)e * D;
-    float acc = 0.f;
-    for (int c = lane; c < D; c += 64) acc += row[c] * rld(wr + c);
-    acc = wave_sum(acc);
-    if (lane == 0) z[e] = acc;
+  if (vec) {
+    // 16-byte loads of the router rows, 4 in flight a lane (D a multiple of the chunk)
+    constexpr int CH = 16 / sizeof(S);
+    const int nch = D / CH;
+    for (int e = wid; e < n + n_gate; e += nw) {
+      const S* wr = W + (long)e * D;
+      float acc = 0.f;
+      for (int c0 = lane; c0 < nch; c0 += 256) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          v[u] = c0 + u * 64 < nch ? *reinterpret_cast<const uint4*>(wr + (long)(c0 + u * 64) * CH)
+                                   : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (c0 + u * 64 >= nch) continue;
+          const float* rr = row + (c0 + u * 64) * CH;
+          if constexpr (sizeof(S) == 2) {
+            float f[8];
+            unpack8bf(v[u], f);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc += rr[q] * f[q];
+          } else {
+            acc += rr[0] * __uint_as_float(v[u].x) + rr[1] * __uint_as_float(v[u].y) +
+                   rr[2] * __uint_as_float(v[u].z) + rr[3] * __uint_as_float(v[u].w);
+          }
+        }
+      }
+      acc = wave_sum(acc);
+      if (lane == 0) z[e] = acc;
+    }
+  } else {
+    for (int e = wid; e < n + n_gate; e += nw) {
+      const S* wr = W + (long)e * D;
+      float acc = 0.f;
+      for (int c = lane; c < D; c += 64) acc += row[c] * rld(wr + c);
+      acc = wave_sum(acc);
+      if (lane == 0) z[e] = acc;
+    }
   }
   __syncthreads();
   if (threadIdx.x != 0) return;
@@ -504,12 +537,13 @@ extern "C" int dli_score_router(float* topk_w, int* topk_ids, float* gates, cons
       (size_t)(D + n + n_gate) * 4 > 60000)
     return (int)hipErrorInvalidValue;
   const size_t sh = (size_t)(D + n + n_gate) * 4;
+  const bool vec = (uintptr_t)W % 16 == 0 && D % (dt == 0 ? 8 : 4) == 0;
   if (dt == 0)
     score_router_kernel<u16><<<T, 256, sh, st>>>(topk_w, topk_ids, gates, (const u16*)h, ldh,
-                                                 (const u16*)W, corr, D, n, n_gate, top);
+                                                 (const u16*)W, corr, D, n, n_gate, top, vec);
   else if (dt == 1)
     score_router_kernel<float><<<T, 256, sh, st>>>(topk_w, topk_ids, gates, (const float*)h, ldh,
-                                                   (const float*)W, corr, D, n, n_gate, top);
+                                                   (const float*)W, corr, D, n, n_gate, top, vec);
   else return (int)hipErrorInvalidValue;
   DLI_RETURN_LAUNCH();
 }
