@@ -119,6 +119,11 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   const int* bt = a.block_tables + (long)s * a.bt_stride;
   const int hpg = H / G, Gk = a.Gk, hpk = H / Gk;
   const int my_p = a.rowmul > 1 ? p0 : p0 + fr;   // this lane's query position (column fr)
+  // key / value heads this workgroup's query heads read: all of them with head mixing, those
+  // of its 8 heads in the wide form (the others are not staged)
+  const int h_last = min(H, hbase + NW) - 1;
+  const int klo = wide ? hbase / hpk : 0, khi = wide ? h_last / hpk + 1 : Gk;
+  const int vlo = wide ? hbase / hpg : 0, vhi = wide ? h_last / hpg + 1 : G;
   const int my_clo = a.chunk > 0 ? my_p / a.chunk * a.chunk : 0;      // first key of its block
   const int clo_last = a.chunk > 0 ? p_last / a.chunk * a.chunk : 0;
   const bool my_q = fr < nq;
@@ -212,8 +217,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
           slot[tid] = j <= p_last ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
         }
       }
-      for (int c0 = 0; c0 < Gk; c0 += CG) {
-        const int cg = min(CG, Gk - c0);
+      for (int c0 = klo; c0 < khi; c0 += CG) {
+        const int cg = min(CG, khi - c0);
         {                                         // this wave's first head of the step: its
           int h0 = -1;                            // query fragments fly with the K tiles
 #pragma unroll
@@ -404,8 +409,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         }
       }
       // O += W' . V per group of kv heads
-      for (int c0 = 0; c0 < G; c0 += CG) {
-        const int cg = min(CG, G - c0);
+      for (int c0 = vlo; c0 < vhi; c0 += CG) {
+        const int cg = min(CG, vhi - c0);
         __syncthreads();                          // Pp complete (first step) / Vt free
         {
           // chunk i = (c * vcpr + ch) * TK + r: consecutive threads take consecutive keys of one

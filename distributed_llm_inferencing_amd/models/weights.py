@@ -189,7 +189,9 @@ def _hybrid_init(name: str, shape: tuple, dev, dtype, seed: int) -> torch.Tensor
     if name.endswith(".shift"):
         return torch.rand(shape, generator=g).to(dev, dtype)
     if name.endswith(".b_in"):
-        return (0.2 * torch.randn(shape, generator=g)).to(dev, dtype)
+        # small: a large value bias is a constant added to every token, which would make a
+        # random-init router send every token to the same experts
+        return (0.02 * torch.randn(shape, generator=g)).to(dev, dtype)
     if name.endswith(".lower"):
         return (0.9 * torch.rand(shape, generator=g)).to(dev, dtype)
     if name.endswith((".f_b", "loop_step")):
