@@ -111,7 +111,10 @@ def run_design_pulunex(a):
             del eng
             torch.cuda.empty_cache()
         for (B, C) in a.design_decode:
+            # the decoded tokens stay inside the block that ends at C: the block mask's worst
+            # case (a nearly full block of keys), not the few keys after a block edge
             n_new = 33
+            C = max(1, C - n_new - 7)
             eng = LLMEngine(cfg, device="cuda:0", max_batch=B, max_model_len=C + n_new + 16,
                             block_size=16, max_kv_tokens=B * (C + n_new + 32) + 4096,
                             max_prefill_tokens=max(8192, C))

@@ -63,6 +63,9 @@ struct MfmaArgs {
   // (latent attention): the launcher presents token t's H heads as H query rows of a
   // one-head problem, all at token t's position: rowmul = H (cu and positions are per token)
   int rowmul;
+  // rows-are-heads with grouped values (the key row is shared by all heads, the values are
+  // not): vrows = heads per value group; row (= head) r applies its weights to group r / vrows
+  int vrows;
   // > 0: the cache rows of the whole window (slot_cap ints) are looked up once at kernel start
   // instead of per key tile (one global round trip and one barrier less per tile)
   int slot_cap;
@@ -117,13 +120,16 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   const int lo = max(max(0, p0 - a.window + 1), a.chunk > 0 ? p0 / a.chunk * a.chunk : 0);
   const int ntiles = (p_last - lo) / TK + 1;
   const int* bt = a.block_tables + (long)s * a.bt_stride;
-  const int hpg = H / G, Gk = a.Gk, hpk = H / Gk;
+  const bool rgrp = a.vrows > 0;
+  const int hpg = rgrp ? 1 : H / G, Gk = a.Gk, hpk = H / Gk;
+  const int row_c = rgrp ? (blockIdx.x * TQ + fr) / a.vrows : 0;   // this lane's row's value group
   const int my_p = a.rowmul > 1 ? p0 : p0 + fr;   // this lane's query position (column fr)
   // key / value heads this workgroup's query heads read: all of them with head mixing, those
   // of its 8 heads in the wide form (the others are not staged)
   const int h_last = min(H, hbase + NW) - 1;
   const int klo = wide ? hbase / hpk : 0, khi = wide ? h_last / hpk + 1 : Gk;
-  const int vlo = wide ? hbase / hpg : 0, vhi = wide ? h_last / hpg + 1 : G;
+  const int vlo = rgrp ? blockIdx.x * TQ / a.vrows : (wide ? hbase / hpg : 0);
+  const int vhi = rgrp ? (blockIdx.x * TQ + nq - 1) / a.vrows + 1 : (wide ? h_last / hpg + 1 : G);
   const int my_clo = a.chunk > 0 ? my_p / a.chunk * a.chunk : 0;      // first key of its block
   const int clo_last = a.chunk > 0 ? p_last / a.chunk * a.chunk : 0;
   const bool my_q = fr < nq;
@@ -452,19 +458,25 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         for (int hh = 0; hh < MAXHW; ++hh) {
           const int h = wide ? hbase + wave : wave + hh * NW;
           if (h >= H) continue;
-          const int c = h / hpg;
-          if (c < c0 || c >= c0 + cg) continue;
           const bf16x8 pf = *reinterpret_cast<const bf16x8*>(
               Pp + ((long)(wide ? wave : h) * TQ + fr) * 40 + fq * 8);
-          const u16* vt = Vt + (long)(c - c0) * dvw * 40;
+          // rows-are-heads with grouped values: every staged group in turn, the weights of
+          // the rows of other groups zeroed (operand B's row is this lane's fr)
+          const int c_lo = rgrp ? c0 : h / hpg, c_hi = rgrp ? c0 + cg : c_lo + 1;
+          if (!rgrp && (c_lo < c0 || c_lo >= c0 + cg)) continue;
+          for (int c = c_lo; c < c_hi; ++c) {
+            bf16x8 pm = pf;
+            if (rgrp && row_c != c) pm = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            const u16* vt = Vt + (long)(c - c0) * dvw * 40;
 #pragma unroll
-          for (int b = 0; b < MAXDVB; ++b) {
-            const int blk = wide ? hh * MAXDVB + b : b;
-            if (blk >= dvb) continue;
-            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (long)(blk * 16 + fr) * 40 + fq * 8);
-            // operand A = V^T rows (dim), operand B = W' rows (query): lane holds dims
-            // blk*16 + 4*fq + r of query fr
-            oacc[hh][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, oacc[hh][b], 0, 0, 0);
+            for (int b = 0; b < MAXDVB; ++b) {
+              const int blk = wide ? hh * MAXDVB + b : b;
+              if (blk >= dvb) continue;
+              const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (long)(blk * 16 + fr) * 40 + fq * 8);
+              // operand A = V^T rows (dim), operand B = W' rows (query): lane holds dims
+              // blk*16 + 4*fq + r of query fr
+              oacc[hh][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pm, oacc[hh][b], 0, 0, 0);
+            }
           }
         }
       }
@@ -576,8 +588,11 @@ static int pick_splits(int num_seqs, int max_seqlen, int H, int dv, int window, 
   const int ndvs = wide ? (dv + 511) / 512 : (dv + 127) / 128, nhs = wide ? (H + NW - 1) / NW : 1;
   const long base = (long)qtiles * num_seqs * ndvs * nhs;
   const int ntiles_max = (window + TQ - 2) / TK + 2;
-  if (base >= 256 || ntiles_max < 4) return 1;
-  long n = 512 / base;
+  if (ntiles_max < 4) return 1;
+  // one-pass (wide) launches that just fill the chip with one workgroup per CU still walk
+  // their tiles one after the other with nothing to hide the staging behind: split them too
+  if (base >= 256 && (!wide || base >= 1024 || ntiles_max < 8)) return 1;
+  long n = (base >= 256 ? 1024 : 512) / base;
   if (n > 16) n = 16;
   if (n > ntiles_max / 2) n = ntiles_max / 2;
   return n < 2 ? 1 : (int)n;
@@ -611,11 +626,12 @@ extern "C" int dli_window_attention_mfma(
   if (chunk < 0 || Gk < 1) return (int)hipErrorInvalidValue;
   // keys a query tile can see: bounds the slot table and the key splits
   const int weff = chunk > 0 && chunk < window ? chunk : window;
-  int rowmul = 1;
+  int rowmul = 1, vrows = 0;
   if (rowhead) {
-    if (talk != nullptr || gate != nullptr || slopes != nullptr || G != 1 || Gk != 1 || max_seqlen != 1 ||
-        ldq != H * dq || ldo != H * dv)
+    if (talk != nullptr || gate != nullptr || slopes != nullptr || Gk != 1 || G < 1 || H % G ||
+        max_seqlen != 1 || ldq != H * dq || ldo != H * dv)
       return (int)hipErrorInvalidValue;
+    if (G > 1) vrows = H / G;   // grouped values under the shared key row
     rowmul = H;            // token t's heads = rows [t*H, (t+1)*H) of a one-head problem
     max_seqlen = H;
     T *= H;
@@ -627,7 +643,7 @@ extern "C" int dli_window_attention_mfma(
                        (uintptr_t)out % 8 == 0 && ldq % 8 == 0 && k_stride % 8 == 0 &&
                        v_stride % 8 == 0 && ldo % 4 == 0;
   const bool wide = talk == nullptr;
-  if (H < 1 || (!wide && H > NW * MAXHW) || G < 1 || H % G || H % Gk || dq % 32 || dv % 16 ||
+  if (H < 1 || (!wide && H > NW * MAXHW) || G < 1 || (vrows == 0 && H % G) || H % Gk || dq % 32 || dv % 16 ||
       !aligned || window < 1 || block_size < 1 || (!wide && Gk != G))
     return (int)hipErrorNotSupported;
   const int dvw = wide ? 512 : 128;
@@ -667,7 +683,7 @@ extern "C" int dli_window_attention_mfma(
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
              H, G, dq, dv, window, scale, Gk, chunk, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
-             slot_cap, nullptr, nullptr, 0};
+             vrows, slot_cap, nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);
     WA_LAUNCH(grid);

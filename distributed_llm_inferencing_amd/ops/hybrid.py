@@ -265,7 +265,7 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
         lib = N.require_native()
         # decode steps of heads that share one cached row per position (latent attention):
         # the heads become the query rows of a one-head problem
-        rowhead = int(G == 1 and H > 1 and int(max_seqlen) == 1 and talk is None and gate is None
+        rowhead = int(Gk == 1 and H > 1 and int(max_seqlen) == 1 and talk is None and gate is None
                       and slopes is None and q.stride(0) == H * dq)
         nb = lib.dli_window_attention_mfma_workspace_bytes(S, int(max_seqlen), T, H, dv,
                                                            int(min(window, chunk) if chunk else window),

@@ -484,7 +484,8 @@ def _paged_case(lens, starts, H, Gk, G, dq, dv, block, seed):
 @pytest.mark.gpu
 @pytest.mark.parametrize("H_,G,dq,dv,size", [(4, 2, 64, 48, 40), (6, 2, 128, 64, 96),
                                              (16, 4, 256, 128, 19), (3, 1, 32, 16, 1),
-                                             (8, 8, 512, 32, 1000), (12, 3, 96, 80, 33)])
+                                             (8, 8, 512, 32, 1000), (12, 3, 96, 80, 33),
+                                             (24, 2, 64, 32, 50), (32, 8, 256, 128, 300)])
 @pytest.mark.parametrize("decode", [False, True])
 def test_matrix_core_attention_with_blocks_and_shared_key_rows(gpu, H_, G, dq, dv, size, decode):
     """The MFMA form with the block mask and one key head per cache row against the PyTorch
