@@ -516,3 +516,29 @@ def test_matrix_core_attention_with_blocks_and_shared_key_rows(gpu, H_, G, dq, d
     assert (scalar - want).abs().max() < lim
     assert (got - want).abs().max() < lim
     assert size == 1 or not torch.equal(got, scalar)      # the two kernels really differ
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("width,lay,n", [
+    (192, layer(heads=6, kv=2, dim=32, vdim=32, size=24,
+                mlp=moe(ff=128, experts=12, identity=4, top=2, shared=64)), 70),
+    (320, layer(heads=5, kv=1, dim=64, vdim=16, size=9,
+                mlp=moe(ff=64, experts=3, identity=1, top=3, shared=0)), 41),
+    (128, layer(heads=2, kv=2, dim=16, vdim=16, size=50, mlp=dense(192)), 33),
+    (64, layer(heads=2, kv=1, dim=32, vdim=32, size=4,
+               mlp=moe(ff=64, experts=2, identity=1, top=2, shared=64)), 1100)],
+    ids=["w192_12experts", "w320_top3", "w128_dense", "long_prompt_2experts"])
+def test_tuned_feed_forward_layout_at_several_sizes(gpu, width, lay, n):
+    """The feed-forwards on the tuned GEMM tiles (fused activation epilogues, grouped expert
+    GEMMs incl. the prompt-sized form) at widths that are multiples of 64 but not powers of
+    two, expert counts that are not, top 3, and single-row decode steps."""
+    c = config([lay, copy.deepcopy(lay)], width=width, vocab=64, positions=1200)
+    c["layers"][1]["mixer"]["kv_from"] = 0
+    w = O.random_weights(c, seed=width)
+    t = toks(n, c["vocab"], 5)
+    want = ref(t, c, w)
+    eng = engine(c, w, "cuda", torch.bfloat16, max_tokens=1280, block_size=16)
+    assert all("ff_tuned" in lp for lp in eng.model.layers)
+    close(replay(eng, t, [n]), want, torch.bfloat16, "whole")
+    if n < 100:
+        close(replay(eng, t, [n - 9, 2] + [1] * 7), want, torch.bfloat16, "portions + decode")
