@@ -66,6 +66,8 @@ struct MfmaArgs {
   // rows-are-heads with grouped values (the key row is shared by all heads, the values are
   // not): vrows = heads per value group; row (= head) r applies its weights to group r / vrows
   int vrows;
+  // value groups staged per apply step (they are packed at their own stride into the K regions)
+  int cgv;
   // > 0: the cache rows of the whole window (slot_cap ints) are looked up once at kernel start
   // instead of per key tile (one global round trip and one barrier less per tile)
   int slot_cap;
@@ -103,9 +105,11 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   u16* Ks = (u16*)smem;                           // [CG][TK][ldk]
   u16* Vt = Ks;                                   // [CG][dvw][40]
   u16* Pm = Ks + CG * max(TK * ldk, dvw * 40) + 512;   // [TQ*TK][Hp] (after 1 KiB of DMA slack)
-  u16* Pp = Pm + (wide ? 0 : TQ * TK * HpS);      // [H][TQ][40] (wide: [NW][TQ][40], by wave)
+  // without head mixing neither the mix operand nor the mixing matrix take LDS
+  const bool lean = wide || a.talk == nullptr;
+  u16* Pp = Pm + (lean ? 0 : TQ * TK * HpS);      // [H][TQ][40] (wide: [NW][TQ][40], by wave)
   u16* Tk = Pp + (wide ? NW : H) * TQ * 40;       // [Hp16][Hp] talk in bf16, zero padded
-  int* slot_all = (int*)(Tk + (wide ? 0 : ((H + 15) & ~15) * Hp));   // [TK] or [slot_cap]
+  int* slot_all = (int*)(Tk + (lean ? 0 : ((H + 15) & ~15) * Hp));   // [TK] or [slot_cap]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
@@ -184,7 +188,10 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   // without head mixing an unsplit launch needs one pass only (see the score phase)
   // (mode 3: one pass per key split; the split's max / sum go out with its un-normalised
   // partial output and the reduce kernel weighs the splits)
-  const bool single = wide && (a.mode == 0 || a.mode == 3);
+  // (the all-heads form, WIDE = false without mixing, runs it too: 4 heads a wave, each with
+  // its own running pair and accumulators, one K staging for every head of the query tile)
+  const bool single = (wide && (a.mode == 0 || a.mode == 3)) || (!wide && lean && a.mode == 0);
+  const auto si = [&](int hh) { return wide ? 0 : hh; };
   const int pass_lo = (a.mode == 2 || single) ? 1 : 0, pass_hi = a.mode == 1 ? 1 : 2;
   const int rowsT = (int)(a.o_ws_stride / ((long)H * dv));   // rows of a partial-output image
   // staging walks: per-thread start indices and 512-chunk strides, divided once
@@ -328,23 +335,25 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
             // one pass (no head mixing, so un-normalised weights can be applied at once):
             // running max with the accumulators rescaled when it moves, 1 / l at the end
             tmax = group4_max(tmax);
-            const float m_new = fmaxf(m_run[0], tmax);
+            const float m_new = fmaxf(m_run[si(hh)], tmax);
             const float mm = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run[0] - mm);
+            const float alpha = __builtin_amdgcn_exp2f(m_run[si(hh)] - mm);
             float w[8];
             float sum = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) { w[i] = __builtin_amdgcn_exp2f(sv[i] - mm); sum += w[i]; }
             sum = group4_sum(sum);
-            l_run[0] = l_run[0] * alpha + sum;
-            m_run[0] = m_new;
+            l_run[si(hh)] = l_run[si(hh)] * alpha + sum;
+            m_run[si(hh)] = m_new;
             if (alpha != 1.f) {
 #pragma unroll
-              for (int g2 = 0; g2 < MAXHW; ++g2)
+              for (int g2 = 0; g2 < MAXHW; ++g2) {
+                if (!wide && g2 != hh) continue;      // this head's accumulators only
 #pragma unroll
                 for (int b = 0; b < MAXDVB; ++b) oacc[g2][b] *= alpha;
+              }
             }
-            u16* dst = Pp + (wave * TQ + fr) * 40 + fq * 4;
+            u16* dst = Pp + ((wide ? wave : h) * TQ + fr) * 40 + fq * 4;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
               uint2 pk;
@@ -415,8 +424,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
         }
       }
       // O += W' . V per group of kv heads
-      for (int c0 = vlo; c0 < vhi; c0 += CG) {
-        const int cg = min(CG, vhi - c0);
+      for (int c0 = vlo; c0 < vhi; c0 += a.cgv) {
+        const int cg = min(a.cgv, vhi - c0);
         __syncthreads();                          // Pp complete (first step) / Vt free
         {
           // chunk i = (c * vcpr + ch) * TK + r: consecutive threads take consecutive keys of one
@@ -517,11 +526,11 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
     }
     return;
   }
-  const float onorm = single ? (l_run[0] > 0.f ? 1.f / l_run[0] : 0.f) : 1.f;
 #pragma unroll
   for (int hh = 0; hh < MAXHW; ++hh) {
     const int h = wide ? hbase + wave : wave + hh * NW;
     if (h >= H) continue;
+    const float onorm = single ? (l_run[si(hh)] > 0.f ? 1.f / l_run[si(hh)] : 0.f) : 1.f;
 #pragma unroll
     for (int b = 0; b < MAXDVB; ++b) {
       const int blk = wide ? hh * MAXDVB + b : b;
@@ -642,9 +651,16 @@ extern "C" int dli_window_attention_mfma(
   const bool aligned = (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 &&
                        (uintptr_t)out % 8 == 0 && ldq % 8 == 0 && k_stride % 8 == 0 &&
                        v_stride % 8 == 0 && ldo % 4 == 0;
-  const bool wide = talk == nullptr;
+  bool wide = talk == nullptr;
+  // every head scores one shared key row (Gk = 1) and the launch is not split over keys: all
+  // heads of a query tile in one workgroup (4 a wave), so the K tile is staged once for them
+  // instead of once per 8 heads
+  if (wide && !rowhead && Gk == 1 && G > 1 && H > NW && H <= NW * MAXHW &&
+      (ws == nullptr || pick_splits(num_seqs, max_seqlen, H, dv, weff, true) == 1))
+    wide = false;
+  const bool lean = talk == nullptr;
   if (H < 1 || (!wide && H > NW * MAXHW) || G < 1 || (vrows == 0 && H % G) || H % Gk || dq % 32 || dv % 16 ||
-      !aligned || window < 1 || block_size < 1 || (!wide && Gk != G))
+      !aligned || window < 1 || block_size < 1 || (talk != nullptr && Gk != G))
     return (int)hipErrorNotSupported;
   const int dvw = wide ? 512 : 128;
   const int Hp = (H + 31) & ~31, Hp16 = (H + 15) & ~15;
@@ -653,7 +669,8 @@ extern "C" int dli_window_attention_mfma(
   int slot_cap = ((weff + TQ - 2) / TK + 2) * TK;
   if ((size_t)slot_cap * 4 > 16 * 1024) slot_cap = 0;
   const size_t fixed = (wide ? (size_t)NW * TQ * 40
-                             : (size_t)TQ * TK * (Hp + 8) + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
+                        : lean ? (size_t)H * TQ * 40
+                               : (size_t)TQ * TK * (Hp + 8) + (size_t)H * TQ * 40 + (size_t)Hp16 * Hp) * 2 +
                        (size_t)(slot_cap > TK ? slot_cap : TK) * 4 + 64 + 1024;
   const size_t per_cg = (size_t)((TK * ldk > dvw * 40) ? TK * ldk : dvw * 40) * 2;
   const size_t budget = 158 * 1024;
@@ -661,6 +678,8 @@ extern "C" int dli_window_attention_mfma(
   int CG = (int)((budget - fixed) / per_cg);
   CG = CG > (G > Gk ? G : Gk) ? (G > Gk ? G : Gk) : CG;
   CG = CG > NW ? NW : CG;
+  int cgv = (int)(CG * (per_cg / 2) / ((size_t)dvw * 40));   // value groups that fit the regions
+  cgv = cgv > G ? G : cgv;
   const size_t sh = fixed + CG * per_cg;
   static bool raised = false;
   if (!raised) {
@@ -679,11 +698,13 @@ extern "C" int dli_window_attention_mfma(
   } while (0)
   const int ndvs = (dv + dvw - 1) / dvw, qtiles = (max_seqlen + TQ - 1) / TQ;
   const int nhs = wide ? (H + NW - 1) / NW : 1;
-  const int nsplit = ws != nullptr ? pick_splits(num_seqs, max_seqlen, H, dv, weff, wide) : 1;
+  // (the all-heads form was chosen because the launch needs no key split)
+  const int nsplit = ws != nullptr && !(lean && !wide)
+                         ? pick_splits(num_seqs, max_seqlen, H, dv, weff, wide) : 1;
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
              H, G, dq, dv, window, scale, Gk, chunk, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
-             vrows, slot_cap, nullptr, nullptr, 0};
+             vrows, cgv, slot_cap, nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);
     WA_LAUNCH(grid);
