@@ -258,6 +258,10 @@ class LLMEngine:
         if self._inflight is not None or self.scheduler.has_work():
             raise RuntimeError("replay_step on an engine with generation requests in flight")
         n_want = sum(len(w) for w in (want or []))
+        if not entries:                     # a step that only ends requests
+            for rid in end:
+                self.scheduler.end_replay(rid)
+            return torch.empty(0, self.cfg.vocab_size, dtype=torch.float32, device=self.device)
         meta = self.scheduler.replay_step(entries, want)
         if n_want == 0:
             meta.logit_rows = np.zeros(1, np.int64)      # the step still runs; row discarded

@@ -378,6 +378,11 @@ def test_first_tokens_and_long_decode(device, dtype):
     close(replay(eng, t, [1, 1, 2, 1] + [1] * 65), want, dtype, "from the first token on")
     close(replay(eng, t[:3], [3]), want[:3], dtype, "three tokens")
     close(replay(eng, t[:1], [1]), want[:1], dtype, "one token")
+    # a request that is ended by a later step which brings no tokens at all
+    lg = eng.replay_step([("z", t[:5])], [[4]], [])
+    assert eng.replay_step([], [], ["z"]).shape[0] == 0
+    close(lg.float().cpu().numpy(), want[4:5], dtype, "ended by an empty step")
+    assert eng.bm.num_free == eng.bm.num_blocks and eng.state_slots.num_free == 4
 
 
 # ------------------------------------------------------------------ generation entry point
